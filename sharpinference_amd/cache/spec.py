@@ -28,10 +28,16 @@ class KVSpec:
     window_kind: int = WINDOW_NONE
     window: int = 0
     v_head_dim: int = 0
+    values_in_keys: bool = False     # the values are a leading part of the key rows: no value tensor is kept
 
     @property
     def value_dim(self) -> int:
         return self.v_head_dim or self.head_dim
+
+    @property
+    def elements_per_token(self) -> int:
+        """Cache elements one token takes in one layer of this kind."""
+        return self.num_kv_heads * (self.head_dim + (0 if self.values_in_keys else self.value_dim))
 
     def first_visible(self, pos: int) -> int:
         """The earliest key position a query at `pos` can see."""

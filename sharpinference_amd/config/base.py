@@ -88,7 +88,9 @@ def architecture_name(d: Dict[str, Any]) -> str:
     archs = d.get("architectures")
     if isinstance(archs, (list, tuple)) and archs and isinstance(archs[0], str):
         return archs[0]
-    raise ConfigError("config.json has no 'architectures' list naming the model class")
+    if isinstance(d.get("architecture"), str) and d["architecture"]:      # some designs name themselves in one string
+        return d["architecture"]
+    raise ConfigError("config.json names no model class ('architectures' list or 'architecture' string)")
 
 
 def load_config(source) -> ModelConfig:

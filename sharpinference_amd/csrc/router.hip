@@ -20,8 +20,16 @@ constexpr int kMaxExperts = 1024;
 
 // One thread: gate the logits g[0 .. n_experts) in place, pick k of them (ascending scan with a
 // strict >, so the lowest index wins a tie) into ids / w.
+// `choice` (or null) is scratch of n_experts + n_groups floats and turns the choice apart from the
+// weights: experts are then picked by g[e] + corr[e] (corr may be null), among the experts of the
+// `keep` best of n_groups equal groups of neighbours only (a group's rank: the sum of its
+// kGroupTop largest choice scores; the lowest index wins a tie; the others' choice scores count as
+// minus infinity), and a pick's weight stays its gate value g[e].
+constexpr int kGroupTop = 2;
+
 __device__ void gate_and_pick(float* g, int n_experts, int k, int gate, int renorm, int* ids, float* w,
-                              float* gate_out) {
+                              float* gate_out, float* choice = nullptr, const float* corr = nullptr,
+                              int n_groups = 1, int keep = 1) {
   if (gate == 0) {
     for (int e = 0; e < n_experts; ++e) g[e] = 1.0f / (1.0f + expf(-g[e]));
   } else {
@@ -37,6 +45,45 @@ __device__ void gate_and_pick(float* g, int n_experts, int k, int gate, int reno
   }
   if (gate_out)
     for (int e = 0; e < n_experts; ++e) gate_out[e] = g[e];
+  const float* by = g;               // what the picks are ranked by
+  if (choice) {
+    for (int e = 0; e < n_experts; ++e) choice[e] = corr ? g[e] + corr[e] : g[e];
+    if (n_groups > 1 && keep < n_groups) {
+      const int per = n_experts / n_groups;
+      float* rank = choice + n_experts;
+      for (int q = 0; q < n_groups; ++q) {
+        // the sum of the group's kGroupTop largest choice scores (of all of them in a smaller group)
+        float top[kGroupTop];
+        for (int i = 0; i < kGroupTop; ++i) top[i] = -INFINITY;
+        for (int e = q * per; e < (q + 1) * per; ++e) {
+          float v = choice[e];
+          for (int i = 0; i < kGroupTop; ++i)
+            if (v > top[i]) {
+              const float o = top[i];
+              top[i] = v;
+              v = o;
+            }
+        }
+        float r = 0.f;
+        for (int i = 0; i < kGroupTop && i < per; ++i) r += top[i];
+        rank[q] = r;
+      }
+      for (int j = 0; j < keep; ++j) {       // the kept groups are marked with +infinity
+        int best = -1;
+        float bv = -INFINITY;
+        for (int q = 0; q < n_groups; ++q)
+          if (rank[q] != INFINITY && (best < 0 || rank[q] > bv)) {
+            bv = rank[q];
+            best = q;
+          }
+        rank[best] = INFINITY;
+      }
+      for (int q = 0; q < n_groups; ++q)
+        if (rank[q] != INFINITY)
+          for (int e = q * per; e < (q + 1) * per; ++e) choice[e] = -INFINITY;
+    }
+    by = choice;
+  }
   float wsum = 0.f;
   for (int j = 0; j < k; ++j) {
     int best = -1;
@@ -44,14 +91,14 @@ __device__ void gate_and_pick(float* g, int n_experts, int k, int gate, int reno
     for (int e = 0; e < n_experts; ++e) {
       bool taken = false;
       for (int i = 0; i < j; ++i) taken |= (ids[i] == e);
-      if (!taken && (best < 0 || g[e] > bv)) {
-        bv = g[e];
+      if (!taken && (best < 0 || by[e] > bv)) {
+        bv = by[e];
         best = e;
       }
     }
     ids[j] = best;
-    w[j] = bv;
-    wsum += bv;
+    w[j] = g[best];
+    wsum += g[best];
   }
   if (renorm && k > 1 && wsum > 0.f)
     for (int j = 0; j < k; ++j) w[j] /= wsum;
@@ -114,9 +161,12 @@ __global__ __launch_bounds__(1024) void router_topk_kernel(const T* __restrict__
                                                            int* __restrict__ topk_ids,
                                                            float* __restrict__ topk_w,
                                                            float* __restrict__ gate_out, int n_tokens, int hidden,
-                                                           int n_experts, int k, int gate, int renorm) {
+                                                           int n_experts, int k, int gate, int renorm,
+                                                           const float* __restrict__ corr, int n_groups, int keep,
+                                                           int split_choice) {
   // TT tokens per block: a router row is fetched once for all of them.
   __shared__ float g[TT][kMaxExperts];
+  extern __shared__ float choice_s[];        // [TT][n_experts + n_groups] when the choice has scores of its own
   const int t0 = blockIdx.x * TT;
   const int lane = threadIdx.x & (kWave - 1);
   const int w = threadIdx.x >> 6;
@@ -136,7 +186,8 @@ __global__ __launch_bounds__(1024) void router_topk_kernel(const T* __restrict__
   if (threadIdx.x < TT && t0 + threadIdx.x < n_tokens) {
     const int t = t0 + threadIdx.x;
     gate_and_pick(g[threadIdx.x], n_experts, k, gate, renorm, topk_ids + (size_t)t * k, topk_w + (size_t)t * k,
-                  gate_out ? gate_out + (size_t)t * n_experts : nullptr);
+                  gate_out ? gate_out + (size_t)t * n_experts : nullptr,
+                  split_choice ? choice_s + (size_t)threadIdx.x * (n_experts + n_groups) : nullptr, corr, n_groups, keep);
   }
 }
 
@@ -226,26 +277,32 @@ SHARPI_EXPORT int sharpi_add_rmsnorm_router(float* h, const void* delta, const v
   return SHARPI_OK;
 }
 
+// corr (float [n_experts] or null): added to the gate values for the choice only.  n_groups, keep:
+// picks come from the `keep` best of n_groups equal groups of neighbouring experts (1, 1: no groups).
 SHARPI_EXPORT int sharpi_router_topk(const void* x, int x_dtype, const void* wr, int w_dtype, int* topk_ids,
                                      float* topk_w, float* gate_out, int n_tokens, int hidden, int n_experts,
-                                     int k, int gate, int renorm, hipStream_t stream) {
+                                     int k, int gate, int renorm, const float* corr, int n_groups, int keep,
+                                     hipStream_t stream) {
   if (n_tokens <= 0) return SHARPI_OK;
   if (hidden <= 0 || n_experts <= 0 || n_experts > kMaxExperts || k <= 0 || k > n_experts) return SHARPI_ERR_ARG;
   if (gate < 0 || gate > 1) return SHARPI_ERR_ARG;
+  if (n_groups < 1 || keep < 1 || keep > n_groups || n_experts % n_groups != 0 || k > keep * (n_experts / n_groups)) return SHARPI_ERR_ARG;
+  const int split_choice = corr != nullptr || keep < n_groups;
   // one wave per expert at a time: enough waves for the experts, at most 16; with many tokens four
   // share a block (and each fetch of a router row)
   const int tt = n_tokens >= 64 ? 4 : 1;
   dim3 grid(ceil_div(n_tokens, tt)), block(kWave * (n_experts >= 16 ? 16 : n_experts >= 8 ? 8 : 4));
+  const size_t lds = split_choice ? (size_t)tt * (n_experts + n_groups) * sizeof(float) : 0;
 #define ROUTER_LAUNCH(TX, TWT)                                                                                   \
   do {                                                                                                           \
     if (tt == 4)                                                                                                 \
-      router_topk_kernel<TX, TWT, 4><<<grid, block, 0, stream>>>((const TX*)x, (const TWT*)wr, topk_ids, topk_w, \
+      router_topk_kernel<TX, TWT, 4><<<grid, block, lds, stream>>>((const TX*)x, (const TWT*)wr, topk_ids, topk_w, \
                                                                  gate_out, n_tokens, hidden, n_experts, k, gate, \
-                                                                 renorm);                                        \
+                                                                 renorm, corr, n_groups, keep, split_choice);    \
     else                                                                                                         \
-      router_topk_kernel<TX, TWT, 1><<<grid, block, 0, stream>>>((const TX*)x, (const TWT*)wr, topk_ids, topk_w, \
+      router_topk_kernel<TX, TWT, 1><<<grid, block, lds, stream>>>((const TX*)x, (const TWT*)wr, topk_ids, topk_w, \
                                                                  gate_out, n_tokens, hidden, n_experts, k, gate, \
-                                                                 renorm);                                        \
+                                                                 renorm, corr, n_groups, keep, split_choice);    \
   } while (0)
   if (x_dtype == DT_F32 && w_dtype == DT_F32) ROUTER_LAUNCH(float, float);
   else if (x_dtype == DT_BF16 && w_dtype == DT_BF16) ROUTER_LAUNCH(bf16_t, bf16_t);

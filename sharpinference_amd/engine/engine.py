@@ -139,7 +139,7 @@ class Engine:
                            None if kv_tokens is None else max(1, (int(kv_tokens) + page_size - 1) // page_size))
         if kv_tokens is None and kv_specs:
             def total_bytes(sz):
-                return sum(sz[s.group_key()] * s.num_kv_heads * (s.head_dim + s.value_dim) * page_size * width for s in kv_specs)
+                return sum(sz[s.group_key()] * s.elements_per_token * page_size * width for s in kv_specs)
             budget = int(torch.cuda.mem_get_info(self.device)[0] * 0.8)
             while total_bytes(sizes) > budget and max(sizes.values()) > 1:
                 big = max(sizes, key=lambda k: sizes[k])       # the largest pools give way first

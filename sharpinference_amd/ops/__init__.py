@@ -389,6 +389,117 @@ def gemm_tiled(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype
 
 
 # ---------------------------------------------------------------------------
+# layers whose norms sit on the branch outputs; latent attention
+# ---------------------------------------------------------------------------
+def norm_add(h: torch.Tensor, delta, weight: torch.Tensor, eps: float,
+             out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """h += unit_rms(delta) * weight, in place in float; with ``out_dtype`` the new h is also
+    returned in that storage type (what the next branch reads).  delta: a tensor [T, H] or an
+    ExpertSum without a shared part (formed on the fly, rounded once to its storage type)."""
+    lazy = delta if isinstance(delta, ExpertSum) else None
+    if lazy is not None and lazy.shared is not None:
+        delta, lazy = lazy.tensor(), None
+    base = lazy.y if lazy is not None else delta
+    _dev(h, base, weight, lazy.weights if lazy is not None else None)
+    _need(h.dim() == 2 and h.dtype == torch.float32, "norm_add: h must be float32 [T, H]")
+    T, H = h.shape
+    _need(tuple(delta.shape) == (T, H), f"norm_add: delta {tuple(delta.shape)} vs h {tuple(h.shape)}")
+    _need(weight.dtype == torch.float32 and weight.shape == (H,), "norm_add: weight must be float32 [H]")
+    if lazy is not None:
+        _need(base.dim() == 2 and base.shape[1] == H, "norm_add: the experts' rows must be [rows, H]")
+    out = torch.empty(T, H, dtype=out_dtype, device=h.device) if out_dtype is not None else None
+    _run("sharpi_norm_add", _ptr(h), _ptr(base), _code(base.dtype), _ptr(weight), _ptr(out),
+         _code(out_dtype) if out_dtype is not None else 0, T, H, float(eps),
+         _ptr(lazy.inv_pos) if lazy is not None else None, _ptr(lazy.weights) if lazy is not None else None,
+         lazy.k if lazy is not None else 0, _stream())
+    return out
+
+
+def latent_prep(proj: torch.Tensor, q_off: int, kv_off: Optional[int], q_full: torch.Tensor,
+                rows: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor], positions: torch.Tensor,
+                inv_freq: Optional[torch.Tensor], norm_w: Optional[torch.Tensor], eps: float, nh: int, dn: int, dr: int,
+                rank: int) -> None:
+    """Per token of proj [T, ld] (queries [nh, dn + dr] at column q_off, the down projection
+    [rank + dr] at column kv_off, None: this layer makes no latent): the rotated query parts go to
+    columns rank.. of every head of q_full [T, nh, rank + dr]; the latent rms_norm(first rank
+    elements) * norm_w and the rotated key part go side by side into the cache rows
+    [pages, 1, page_size, rank + dr] at slot_mapping (-1: nothing stored).  inv_freq float32
+    [pairs]: pairs (2i, 2i + 1) of the rotated parts turn by position * inv_freq[i]."""
+    _dev(proj, q_full, rows, slot_mapping, positions, inv_freq, norm_w)
+    _i32(slot_mapping, "slot_mapping")
+    _i32(positions, "positions")
+    T, ld = proj.shape
+    D = rank + dr
+    _need(q_full.shape == (T, nh * D) and q_full.dtype == proj.dtype, "latent_prep: q_full must be [T, nh * (rank + dr)] of proj's dtype")
+    _need(positions.shape == (T,), "latent_prep: positions must be [T]")
+    n_pairs = 0
+    if inv_freq is not None:
+        _need(inv_freq.dtype == torch.float32 and inv_freq.dim() == 1 and 2 * inv_freq.shape[0] <= dr,
+              "latent_prep: inv_freq must be float32 [pairs], 2 * pairs <= dr")
+        n_pairs = inv_freq.shape[0]
+    if kv_off is not None:
+        _need(rows is not None and rows.dim() == 4 and rows.shape[1] == 1 and rows.shape[3] == D and rows.dtype == proj.dtype,
+              "latent_prep: cache rows must be [pages, 1, page_size, rank + dr] of proj's dtype")
+        _need(slot_mapping is not None and slot_mapping.shape == (T,), "latent_prep: slot_mapping must be [T]")
+        _need(norm_w is not None and norm_w.dtype == torch.float32 and norm_w.shape == (rank,), "latent_prep: norm_w must be float32 [rank]")
+    _run("sharpi_latent_prep", _ptr(proj), _code(proj.dtype), ld, int(q_off), -1 if kv_off is None else int(kv_off),
+         _ptr(q_full), _ptr(rows) if kv_off is not None else None, _ptr(slot_mapping) if kv_off is not None else None,
+         _ptr(positions), _ptr(inv_freq), n_pairs, _ptr(norm_w) if kv_off is not None else None, float(eps), T, nh, dn, dr,
+         rank, _stream())
+
+
+def head_gemm(x: torch.Tensor, x_off: int, sx: int, w: torch.Tensor, out: torch.Tensor, out_off: int, so: int,
+              gate: Optional[torch.Tensor] = None, gate_off: int = 0) -> torch.Tensor:
+    """One product per head: out[t, out_off + h * so + n] = sum_k x[t, x_off + h * sx + k] * w[h, n, k]
+    for w [nh, N, K], times sigmoid(gate[t, gate_off + h * N + n]) where a gate is given.  x, out and
+    gate are rows of one storage type; every sum is one float chain in ascending k."""
+    _dev(x, w, out, gate)
+    _need(x.dim() == 2 and out.dim() == 2 and w.dim() == 3 and x.shape[0] == out.shape[0], "head_gemm: x [T, ..], out [T, ..], w [nh, N, K]")
+    nh, N, K = w.shape
+    _need(x.dtype == w.dtype == out.dtype and (gate is None or gate.dtype == x.dtype), "head_gemm: one storage type for all operands")
+    ldx, ldo = x.shape[1], out.shape[1]
+    _need(x_off >= 0 and sx >= K and x_off + (nh - 1) * sx + K <= ldx, "head_gemm: the heads' inputs do not fit x")
+    _need(out_off >= 0 and so >= N and out_off + (nh - 1) * so + N <= ldo, "head_gemm: the heads' outputs do not fit out")
+    width = x.element_size()
+    gp, ldg = None, 0
+    if gate is not None:
+        _need(gate.dim() == 2 and gate.shape[0] == x.shape[0] and gate_off >= 0 and gate_off + nh * N <= gate.shape[1],
+              "head_gemm: the gate does not fit")
+        gp, ldg = gate.data_ptr() + gate_off * width, gate.shape[1]
+    _run("sharpi_head_gemm", x.data_ptr() + x_off * width, _code(x.dtype), ldx, sx, _ptr(w),
+         out.data_ptr() + out_off * width, ldo, so, gp, ldg, x.shape[0], nh, N, K, _stream())
+    return out
+
+
+LATENT_MAX_RANK = 512    # the latent attention kernels hold this many value elements a row
+
+
+def attention_latent(q: torch.Tensor, rows: torch.Tensor, group, ctx, scale: float, nh: int, rank: int, dr: int,
+                     sink: Optional[torch.Tensor] = None, window_kind: int = WINDOW_NONE, window: int = 0) -> torch.Tensor:
+    """Attention of nh query heads over one shared cache row per key (rows [pages, 1, page_size,
+    rank + dr]): score = scale * q . row over all rank + dr elements, value = the row's first rank
+    elements, softmax in float with exp(sink[h]) as one more term of the denominator where sinks
+    (float32 [nh]) are given.  q [T, nh * (rank + dr)] -> [T, nh * rank]."""
+    _dev(q, rows, group.block_table, ctx.entry_of_token, ctx.positions, sink)
+    T = q.shape[0]
+    D = rank + dr
+    _need(q.shape == (T, nh * D), "attention_latent: q must be [T, nh * (rank + dr)]")
+    _need(rows.dim() == 4 and rows.shape[1] == 1 and rows.shape[3] == D and rows.dtype == q.dtype,
+          "attention_latent: cache rows must be [pages, 1, page_size, rank + dr] of q's dtype")
+    _need(1 <= rank <= LATENT_MAX_RANK, f"attention_latent: a latent of {rank} is not taken (1 to {LATENT_MAX_RANK})")
+    if sink is not None:
+        _need(sink.dtype == torch.float32 and sink.shape == (nh,), "attention_latent: sink must be float32 [nh]")
+    _i32(group.block_table, "block_table")
+    _need(group.block_table.dim() == 2 and ctx.entry_of_token.shape == (T,) and ctx.positions.shape == (T,),
+          "attention_latent: block_table [entries, max_blocks], per-token arrays [T]")
+    out = torch.empty(T, nh * rank, dtype=q.dtype, device=q.device)
+    _run("sharpi_attention_latent", _ptr(q), _ptr(rows), _code(q.dtype), _ptr(group.block_table), _ptr(ctx.entry_of_token),
+         _ptr(ctx.positions), _ptr(sink), _ptr(out), int(window_kind), int(window), float(scale), T, nh, rank, dr,
+         rows.shape[2], group.block_table.shape[1], rows.shape[0], _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------
 # weights stored for streaming
 # ---------------------------------------------------------------------------
 class PackedWeight:
@@ -705,18 +816,27 @@ GATE_SIGMOID, GATE_SOFTMAX = 0, 1
 
 
 def router_topk(x: torch.Tensor, wr: torch.Tensor, k: int, gate: int = GATE_SIGMOID, renorm: bool = False,
-                want_gates: bool = False):
+                want_gates: bool = False, correction: Optional[torch.Tensor] = None, n_groups: int = 1,
+                keep_groups: int = 1):
     """Router logits in float, gate, k picks (lowest index wins a tie).
-    Returns ids int32 [T, k], weights float32 [T, k] (and the gate values [T, E] if asked)."""
-    _dev(x, wr)
+    Returns ids int32 [T, k], weights float32 [T, k] (and the gate values [T, E] if asked).
+    ``correction`` (float32 [E]) is added to the gate values for the choice only: the weights stay
+    the gate values.  With ``n_groups`` > ``keep_groups`` the experts form n_groups equal groups of
+    neighbours and only those of the keep_groups best groups can be picked (a group's rank: the sum
+    of its two largest choice scores)."""
+    _dev(x, wr, correction)
     _need(x.dim() == 2 and wr.dim() == 2 and x.shape[1] == wr.shape[1], "router: x [T, H], wr [E, H]")
     T, H = x.shape
     E = wr.shape[0]
+    if correction is not None:
+        _need(correction.dtype == torch.float32 and correction.shape == (E,), "router: correction must be float32 [E]")
+    _need(1 <= keep_groups <= n_groups and E % n_groups == 0 and k <= keep_groups * (E // n_groups),
+          f"router: {n_groups} groups (keep {keep_groups}) do not fit {E} experts and {k} picks")
     ids = torch.empty(T, k, dtype=torch.int32, device=x.device)
     wts = torch.empty(T, k, dtype=torch.float32, device=x.device)
     gates = torch.empty(T, E, dtype=torch.float32, device=x.device) if want_gates else None
     _run("sharpi_router_topk", _ptr(x), _code(x.dtype), _ptr(wr), _code(wr.dtype), _ptr(ids), _ptr(wts), _ptr(gates),
-         T, H, E, k, gate, 1 if renorm else 0, _stream())
+         T, H, E, k, gate, 1 if renorm else 0, _ptr(correction), int(n_groups), int(keep_groups), _stream())
     return (ids, wts, gates) if want_gates else (ids, wts)
 
 
@@ -806,9 +926,10 @@ def moe_permute(ids: torch.Tensor, wts: torch.Tensor, n_experts: int, shared_gro
 
 
 def route(x: torch.Tensor, wr: torch.Tensor, k: int, gate: int = GATE_SIGMOID, renorm: bool = False,
-          shared_group: bool = False):
+          shared_group: bool = False, correction: Optional[torch.Tensor] = None, n_groups: int = 1,
+          keep_groups: int = 1):
     """router_topk then moe_permute: (ids, weights, Routing)."""
-    ids, wts = router_topk(x, wr, k, gate, renorm)
+    ids, wts = router_topk(x, wr, k, gate, renorm, correction=correction, n_groups=n_groups, keep_groups=keep_groups)
     return ids, wts, moe_permute(ids, wts, wr.shape[0], shared_group)
 
 

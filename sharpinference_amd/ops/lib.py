@@ -36,7 +36,11 @@ _SIGNATURES = {
     "sharpi_gemm_skinny_swiglu": [P, P, P, I, I, I, P, P, I, P, I, I, I, I, I, P],
     "sharpi_gemm_skinny_picked": [P, P, P, I, I, I, P, P, I, I, I, I, I, I, I, I, I, P],
     "sharpi_add_rmsnorm_router": [P, P, P, I, P, I, I, F, P, I, P, P, I, I, I, I, P],
-    "sharpi_router_topk": [P, I, P, I, P, P, P, I, I, I, I, I, I, P],
+    "sharpi_router_topk": [P, I, P, I, P, P, P, I, I, I, I, I, I, P, I, I, P],
+    "sharpi_norm_add": [P, P, I, P, P, I, I, I, F, P, P, I, P],
+    "sharpi_latent_prep": [P, I, I, I, I, P, P, P, P, P, I, P, F, I, I, I, I, I, P],
+    "sharpi_head_gemm": [P, I, I, I, P, P, I, I, P, I, I, I, I, I, P],
+    "sharpi_attention_latent": [P, P, I, P, P, P, P, P, I, I, F, I, I, I, I, I, I, I, P],
     "sharpi_moe_permute": [P, P, P, P, P, P, P, I, I, I, I, I, P],
     "sharpi_gemm_grouped": [P, I, P, P, I, I, I, I, P, P, P, I, I, I, P],
     "sharpi_gemm_grouped_swiglu": [P, I, P, P, I, I, I, P, P, P, I, P, I, I, I, P],

@@ -126,6 +126,7 @@ class ResidualStream:
     def __init__(self, h: torch.Tensor):
         self.h = h
         self.pending = None
+        self.act = None        # h in the activations' storage type, where a block keeps such a copy beside it
 
     def pending_tensor(self) -> Optional[torch.Tensor]:
         p = self.pending

@@ -3,6 +3,9 @@ from __future__ import annotations
 
 from typing import Dict
 
+import torch
+
+from .. import ops
 from .base import LayerCache, ParamSpec, Part, ResidualStream, StepContext, TensorSource
 
 
@@ -61,3 +64,36 @@ class PreNormBlock(Part):
         else:
             n = self.norm2.forward(stream, ctx.act_dtype)
             stream.pending = self.ffn.forward(n, ctx)
+
+
+class PostNormBlock(PreNormBlock):
+    """h += norm1(mixer(h)); h += norm2(ffn(h)): the branches read the residual sum itself and the
+    norms sit on their outputs.  ``ffn`` None: a layer of a mixer alone.  The sum stays float; a
+    branch reads it in the activations' storage type, a copy that the norm kernel leaves beside
+    the sum (``stream.act``; the sum itself in float32), so a layer costs no launch for it."""
+
+    def __init__(self, norm1: Part, mixer: Part, norm2: Part = None, ffn: Part = None, names=None):
+        if (norm2 is None) != (ffn is None):
+            raise ValueError("a feed-forward and its norm come together")
+        super().__init__(norm1, mixer, norm2, ffn, names or {"norm1": "norm1.", "mixer": "mixer.", "norm2": "norm2.", "ffn": "ffn."})
+
+    def _children(self):
+        kids = [(self.names["norm1"], self.norm1), (self.names["mixer"], self.mixer)]
+        if self.ffn is not None:
+            kids += [(self.names["norm2"], self.norm2), (self.names["ffn"], self.ffn)]
+        return tuple(kids)
+
+    @staticmethod
+    def _input(stream: ResidualStream, ctx: StepContext) -> torch.Tensor:
+        if stream.pending is not None:
+            raise ValueError("a block with norms on its outputs cannot follow one that leaves its output pending")
+        if stream.act is None or stream.act.dtype != ctx.act_dtype:
+            stream.act = stream.h if ctx.act_dtype == torch.float32 else ops.cast(stream.h, ctx.act_dtype)
+        return stream.act
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: LayerCache) -> None:
+        y = self.mixer.forward(self._input(stream, ctx), ctx, cache)
+        self.norm1.add_normed(stream, y, ctx.act_dtype)
+        if self.ffn is not None:
+            y = self.ffn.forward(stream.act, ctx)
+            self.norm2.add_normed(stream, y, ctx.act_dtype)

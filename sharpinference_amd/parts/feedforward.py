@@ -88,9 +88,26 @@ class MoESwiGLU(Part):
                                    # product; off: measured at 2,048 tokens, 1.48 ms a layer against 0.93 + 0.45 with
                                    # the library's product for the shared expert (which runs at the matrix cores' peak)
 
+    NAMES = {"router": "router.weight", "gate": "experts.gate_proj", "up": "experts.up_proj",
+             "down": "experts.down_proj", "shared": "shared_expert.", "correction": "router.correction"}
+
     def __init__(self, hidden: int, num_experts: int, top_k: int, expert_intermediate: int,
                  shared_intermediate: Optional[int] = None, gate: str = "sigmoid", renormalise: bool = False,
-                 score_on_input: bool = True, activation: str = "silu"):
+                 score_on_input: bool = True, activation: str = "silu", correction: bool = False,
+                 n_groups: int = 1, keep_groups: int = 1, names: Optional[Dict[str, str]] = None):
+        """``correction``: a stored vector [E] is added to the gate values where experts are chosen
+        (the weights stay the gate values).  ``n_groups`` / ``keep_groups``: the experts form
+        n_groups equal groups of neighbours and are chosen from the keep_groups best of them only
+        (a group's rank: the sum of its two largest choice scores).  ``names``: the tensors' names
+        behind the part's prefix; a gate / up / down name with ``{e}`` in it is one matrix per
+        expert (stacked when loaded) instead of one stacked tensor."""
+        self.names = {**self.NAMES, **(names or {})}
+        self.correction = bool(correction)
+        self.n_groups, self.keep_groups = int(n_groups), int(keep_groups)
+        if not (1 <= self.keep_groups <= self.n_groups and num_experts % self.n_groups == 0
+                and top_k <= self.keep_groups * (num_experts // self.n_groups)):
+            raise ValueError(f"{n_groups} groups of which {keep_groups} are kept do not fit {num_experts} experts and {top_k} picks")
+        self.w_correction: Optional[torch.Tensor] = None
         if not 1 <= top_k <= num_experts:
             raise ValueError(f"top_k {top_k} must lie in 1..{num_experts}")
         if num_experts > ops.ROUTER_MAX_EXPERTS:
@@ -108,26 +125,48 @@ class MoESwiGLU(Part):
         self.w_gate_up: Optional[torch.Tensor] = None     # [E, 2*I, H]
         self.w_down: Optional[torch.Tensor] = None        # [E, H, I]
 
-    def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
-        out = {
-            prefix + "router.weight": ParamSpec((self.E, self.hidden)),
-            prefix + "experts.gate_proj": ParamSpec((self.E, self.inter, self.hidden)),
-            prefix + "experts.up_proj": ParamSpec((self.E, self.inter, self.hidden)),
-            prefix + "experts.down_proj": ParamSpec((self.E, self.hidden, self.inter)),
-        }
-        if self.shared is not None:
-            out.update(self.shared.param_specs(prefix + "shared_expert."))
+    def _expert_specs(self, prefix: str, which: str, shape) -> Dict[str, ParamSpec]:
+        name = self.names[which]
+        if "{e}" in name:
+            return {prefix + name.format(e=e): ParamSpec(tuple(shape)) for e in range(self.E)}
+        return {prefix + name: ParamSpec((self.E, *shape))}
+
+    def _expert_stack(self, prefix: str, which: str, source: TensorSource) -> torch.Tensor:
+        name = self.names[which]
+        if "{e}" not in name:
+            return source.get(prefix + name)
+        first = source.get(prefix + name.format(e=0))
+        out = torch.empty((self.E, *first.shape), dtype=first.dtype, device=first.device)
+        out[0].copy_(first)
+        for e in range(1, self.E):
+            out[e].copy_(source.get(prefix + name.format(e=e)))
         return out
 
+    def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
+        out = {prefix + self.names["router"]: ParamSpec((self.E, self.hidden))}
+        out.update(self._expert_specs(prefix, "gate", (self.inter, self.hidden)))
+        out.update(self._expert_specs(prefix, "up", (self.inter, self.hidden)))
+        out.update(self._expert_specs(prefix, "down", (self.hidden, self.inter)))
+        if self.correction:
+            out[prefix + self.names["correction"]] = ParamSpec((self.E,))
+        if self.shared is not None:
+            out.update(self.shared.param_specs(prefix + self.names["shared"]))
+        return out
+
+    def _route_args(self) -> dict:
+        return dict(correction=self.w_correction, n_groups=self.n_groups, keep_groups=self.keep_groups)
+
     def load(self, prefix: str, source: TensorSource) -> None:
-        self.w_router = source.get(prefix + "router.weight")
-        g = source.get(prefix + "experts.gate_proj")
-        u = source.get(prefix + "experts.up_proj")
-        d = source.get(prefix + "experts.down_proj")
+        self.w_router = source.get(prefix + self.names["router"])
+        if self.correction:
+            self.w_correction = source.get(prefix + self.names["correction"]).float().contiguous()
+        g = self._expert_stack(prefix, "gate", source)
+        u = self._expert_stack(prefix, "up", source)
+        d = self._expert_stack(prefix, "down", source)
         self.merged = False
         sh = self.shared
         if sh is not None:
-            sh.load(prefix + "shared_expert.", source)
+            sh.load(prefix + self.names["shared"], source)
         bf16 = g.dtype == u.dtype == d.dtype == torch.bfloat16
         # The experts' matrices are kept only in the order the kernels stream them (no rows: both
         # the few-rows and the many-rows product of the experts read that order), if the sizes allow.
@@ -202,7 +241,8 @@ class MoESwiGLU(Part):
         """The block's second half from the residual stream: normalise and feed forward.  With a
         few decode tokens the norm and the router are one launch (the bits of the two)."""
         T = stream.h.shape[0]
-        if (self._few_tokens(T, ctx) and isinstance(norm, RMSNorm)
+        plain_choice = self.w_correction is None and self.keep_groups == self.n_groups   # what the fused kernel picks by
+        if (self._few_tokens(T, ctx) and isinstance(norm, RMSNorm) and plain_choice
                 and ops.norm_router_ok(stream.h, stream.pending, ctx.act_dtype)):
             with section("norm + router", nbytes=T * self.hidden * 10 + 2 * self.E * self.hidden):
                 x, ids, wts = ops.add_rmsnorm_router(stream.h, stream.pending, norm.weight, norm.eps, self.w_router, self.k,
@@ -216,12 +256,13 @@ class MoESwiGLU(Part):
         trace = ctx.extras.get("router_trace")
         if self._few_tokens(T, ctx):
             with section("router", nbytes=2 * T * self.hidden + 2 * self.E * self.hidden):
-                ids, wts = ops.router_topk(x, self.w_router, self.k, self.gate, self.renormalise)
+                ids, wts = ops.router_topk(x, self.w_router, self.k, self.gate, self.renormalise, **self._route_args())
             return self._picked(x, ids, wts, ctx)
         many = self.MERGE_MIN_MANY_TOKENS is not None and T >= self.MERGE_MIN_MANY_TOKENS
         merge = self.merged and ctx.act_dtype == torch.bfloat16 and (T <= self.MERGE_MAX_TOKENS or many)
         with section("router", nbytes=2 * T * self.hidden + 2 * self.E * self.hidden):
-            ids, wts, rt = ops.route(x, self.w_router, self.k, self.gate, self.renormalise, shared_group=merge)
+            ids, wts, rt = ops.route(x, self.w_router, self.k, self.gate, self.renormalise, shared_group=merge,
+                                     **self._route_args())
         if trace is not None:      # the picks of this step, layer by layer (reference: ForwardPass.cs:2042-2056)
             trace.append((ids, wts, x))
         after = None if self.score_on_input else wts     # scores applied where the outputs are summed

@@ -16,16 +16,31 @@ class RMSNorm(Part):
     src/SharpInference.Cuda/CudaTextKernels.cs:199-224).  ``has_weight=False`` is the
     weightless form (SimdKernels.cs:4252-4283)."""
 
-    def __init__(self, dim: int, eps: float, has_weight: bool = True):
+    def __init__(self, dim: int, eps: float, has_weight: bool = True, name: str = "weight"):
         self.dim, self.eps, self.has_weight = int(dim), float(eps), bool(has_weight)
+        self.name = name           # the weight's name behind the part's prefix ("" : the prefix is the name)
         self.weight: Optional[torch.Tensor] = None
+        self._weight_f32: Optional[torch.Tensor] = None
 
     def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
-        return {prefix + "weight": ParamSpec((self.dim,), INIT_NORM_WEIGHT)} if self.has_weight else {}
+        return {prefix + self.name: ParamSpec((self.dim,), INIT_NORM_WEIGHT)} if self.has_weight else {}
 
     def load(self, prefix: str, source: TensorSource) -> None:
         if self.has_weight:
-            self.weight = source.get(prefix + "weight")
+            self.weight = source.get(prefix + self.name)
+            self._weight_f32 = None
+
+    def add_normed(self, stream: ResidualStream, delta, out_dtype: Optional[torch.dtype]) -> None:
+        """The norm on a branch's output: h += unit_rms(delta) * w in float (delta a tensor or a
+        sum of experts' rows still to be formed), and ``stream.act`` = the new h in ``out_dtype``
+        (h itself where that is float32: no copy is made)."""
+        if self._weight_f32 is None:
+            self._weight_f32 = self.weight.float().contiguous() if self.has_weight else \
+                torch.ones(self.dim, dtype=torch.float32, device=stream.h.device)
+        copy = out_dtype is not None and out_dtype != torch.float32
+        with section("norm", nbytes=stream.h.shape[0] * self.dim * 12):
+            out = ops.norm_add(stream.h, delta, self._weight_f32, self.eps, out_dtype if copy else None)
+        stream.act = out if copy else stream.h
 
     def forward(self, stream: ResidualStream, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Fold the pending branch output into the residual sum and normalise.  With ``rows``

@@ -61,4 +61,4 @@ def _ensure_builtin() -> None:
     if _builtin_done:
         return
     _builtin_done = True
-    from .models import llama4  # noqa: F401  (registers itself)
+    from .models import kuvonex, llama4  # noqa: F401  (register themselves)
