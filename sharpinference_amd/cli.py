@@ -74,7 +74,7 @@ def parse_device(text: Optional[str]) -> str:
 
 
 def build_parser() -> argparse.ArgumentParser:
-    ap = argparse.ArgumentParser(prog="sharpi-cli", description="Generate with a Llama 4 model folder on one MI355X.")
+    ap = argparse.ArgumentParser(prog="sharpi-cli", description="Generate with a model folder (any registered architecture) on one MI355X.")
     ap.add_argument("-m", "--model", required=True, help="model folder (config.json, model.safetensors)")
     ap.add_argument("-p", "--prompt", help="prompt: text (the folder's tokenizer.json encodes it) or token ids "
                                            "(comma or space separated numbers)")

@@ -116,13 +116,15 @@ def latent_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], p: str, mx: di
     return o @ w[p + "o"].T, kept
 
 
-def route(h: torch.Tensor, w_router: torch.Tensor, correction: torch.Tensor, router: dict):
-    """Picks and weights.  s = sigmoid(W_router h); experts are chosen by s + correction, among
+def route(h: torch.Tensor, w_router: torch.Tensor, correction: torch.Tensor, router: dict, ids=None):
+    """Picks and weights (`ids` given: only the weights of those picks are made).  s = sigmoid(W_router h); experts are chosen by s + correction, among
     the experts of the `keep` best groups only (a group's rank: the sum of its GROUP_TOP largest
     choice scores); the weights are s of the chosen, as they are.  Returns ids [T, top] (best
     first), weights [T, top]."""
     E, top = int(router["experts"]), int(router["top"])
-    s = torch.sigmoid(h.to(torch.float32) @ w_router.to(torch.float32).T).to(h.dtype)
+    s = torch.sigmoid(h @ w_router.T)
+    if ids is not None:
+        return ids, s.gather(1, ids)
     choice = s + correction
     groups = router.get("groups")
     if groups:
@@ -143,8 +145,9 @@ def expert(h: torch.Tensor, w: Dict[str, torch.Tensor], p: str) -> torch.Tensor:
 
 
 def moe(h: torch.Tensor, w: Dict[str, torch.Tensor], p: str, mlp: dict, picks=None) -> torch.Tensor:
-    """The weighted sum of the chosen experts' outputs (`picks` = (ids, weights) replaces the router's)."""
-    ids, wts = picks if picks is not None else route(h, w[p + "router"], w[p + "correction"], mlp["router"])
+    """The weighted sum of the chosen experts' outputs (`picks`: expert ids [T, top] that replace the
+    router's choice; their weights are still the router's scores)."""
+    ids, wts = route(h, w[p + "router"], w[p + "correction"], mlp["router"], picks)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, s in zip(ids[t].tolist(), wts[t]):
@@ -159,7 +162,7 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens: Sequence[int], picks:
             want_layers: bool = False):
     """Logits [T, vocab] of a whole sequence (and the residual stream after every layer, if asked).
     A layer is x += norm1(mixer(x)); x += norm2(ff(x)): the branches read x itself, the norms sit
-    on their outputs.  `picks` {layer: (ids, weights)} replaces the routers' choices."""
+    on their outputs.  `picks` {layer: ids [T, top]} replaces the routers' choices."""
     eps = float(cfg["norm"]["eps"])
     x = embed(tokens, w["embed"], float(cfg["embedding"]["scale"]))
     pos = torch.arange(len(tokens))
