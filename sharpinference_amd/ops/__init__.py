@@ -474,12 +474,36 @@ def head_gemm(x: torch.Tensor, x_off: int, sx: int, w: torch.Tensor, out: torch.
 LATENT_MAX_RANK = 512    # the latent attention kernels hold this many value elements a row
 
 
+LATENT_DECODE_RUN_KEYS = 256     # keys a block of the matrix-core latent kernel walks in steps of single tokens
+LATENT_PROMPT_RUN_KEYS = 1024    # ... at least, in steps with prompt portions (at most two runs a row)
+
+
+def latent_run_keys(max_context: int, prompt_step: bool) -> int:
+    """Keys per run of the matrix-core latent attention kernel.  Runs start at multiples of this,
+    whatever the batch.  Steps of single tokens take short runs (many blocks for few rows); steps
+    with prompt portions take runs of at least half the longest context, so that a row has at most
+    two and the scratch for unmerged runs stays small."""
+    if not prompt_step:
+        return LATENT_DECODE_RUN_KEYS
+    run = LATENT_PROMPT_RUN_KEYS
+    while 2 * run < max_context:
+        run *= 2
+    return run
+
+
+def latent_mfma_ok(dtype: torch.dtype, rank: int, dr: int, window_kind: int = WINDOW_NONE) -> bool:
+    return dtype == torch.bfloat16 and window_kind == WINDOW_NONE and _lib.latent_attention_takes(rank, dr)
+
+
 def attention_latent(q: torch.Tensor, rows: torch.Tensor, group, ctx, scale: float, nh: int, rank: int, dr: int,
-                     sink: Optional[torch.Tensor] = None, window_kind: int = WINDOW_NONE, window: int = 0) -> torch.Tensor:
+                     sink: Optional[torch.Tensor] = None, window_kind: int = WINDOW_NONE, window: int = 0,
+                     kernel: Optional[str] = None) -> torch.Tensor:
     """Attention of nh query heads over one shared cache row per key (rows [pages, 1, page_size,
     rank + dr]): score = scale * q . row over all rank + dr elements, value = the row's first rank
     elements, softmax in float with exp(sink[h]) as one more term of the denominator where sinks
-    (float32 [nh]) are given.  q [T, nh * (rank + dr)] -> [T, nh * rank]."""
+    (float32 [nh]) are given.  q [T, nh * (rank + dr)] -> [T, nh * rank].  bfloat16 rows of sizes
+    the matrix-core kernel takes go there (prompt tiles and single tokens from the step's work
+    lists, runs merged afterwards); everything else, and ``kernel="generic"``, through the float kernel."""
     _dev(q, rows, group.block_table, ctx.entry_of_token, ctx.positions, sink)
     T = q.shape[0]
     D = rank + dr
@@ -493,6 +517,30 @@ def attention_latent(q: torch.Tensor, rows: torch.Tensor, group, ctx, scale: flo
     _need(group.block_table.dim() == 2 and ctx.entry_of_token.shape == (T,) and ctx.positions.shape == (T,),
           "attention_latent: block_table [entries, max_blocks], per-token arrays [T]")
     out = torch.empty(T, nh * rank, dtype=q.dtype, device=q.device)
+    mfma = latent_mfma_ok(q.dtype, rank, dr, window_kind) and (ctx.n_decode or ctx.n_prefill_tiles) and group.max_context > 0
+    _need(kernel in (None, "generic", "mfma") and (kernel != "mfma" or mfma), "attention_latent: this step cannot take the kernel asked for")
+    if mfma and kernel != "generic":
+        run = latent_run_keys(group.max_context, bool(ctx.n_prefill_tiles))
+        max_runs = (group.max_context + run - 1) // run
+        part_o = part_ml = None
+        if max_runs > 1:
+            part_o = torch.empty(T * nh * max_runs * rank, dtype=torch.float32, device=q.device)
+            part_ml = torch.empty(T * nh * max_runs * 2, dtype=torch.float32, device=q.device)
+        common = (_ptr(sink), _ptr(out), _ptr(part_o), _ptr(part_ml), float(scale), nh, rank, dr, run, max_runs,
+                  rows.shape[2], group.block_table.shape[1], rows.shape[0], _stream())
+        if ctx.n_prefill_tiles:
+            _i32(ctx.prefill_tiles, "tiles")
+            _need(ctx.prefill_tiles.dim() == 2 and ctx.prefill_tiles.shape[1] == 3, "attention_latent: tiles [n, 3]")
+            _run("sharpi_attention_latent_mfma", _ptr(q), _ptr(rows), _ptr(group.block_table), _ptr(ctx.entry_of_token),
+                 _ptr(ctx.positions), _ptr(ctx.prefill_tiles), None, ctx.prefill_tiles.shape[0], int(ctx.prefill_tile_tokens), *common)
+        if ctx.n_decode:
+            _i32(ctx.decode_tokens, "decode_tokens")
+            _run("sharpi_attention_latent_mfma", _ptr(q), _ptr(rows), _ptr(group.block_table), _ptr(ctx.entry_of_token),
+                 _ptr(ctx.positions), None, _ptr(ctx.decode_tokens), int(ctx.n_decode), 0, *common)
+        if max_runs > 1:
+            _run("sharpi_attention_latent_merge", _ptr(part_o), _ptr(part_ml), _ptr(ctx.positions), None, T, _ptr(sink),
+                 _ptr(out), nh, rank, run, max_runs, _stream())
+        return out
     _run("sharpi_attention_latent", _ptr(q), _ptr(rows), _code(q.dtype), _ptr(group.block_table), _ptr(ctx.entry_of_token),
          _ptr(ctx.positions), _ptr(sink), _ptr(out), int(window_kind), int(window), float(scale), T, nh, rank, dr,
          rows.shape[2], group.block_table.shape[1], rows.shape[0], _stream())

@@ -41,6 +41,8 @@ _SIGNATURES = {
     "sharpi_latent_prep": [P, I, I, I, I, P, P, P, P, P, I, P, F, I, I, I, I, I, P],
     "sharpi_head_gemm": [P, I, I, I, P, P, I, I, P, I, I, I, I, I, P],
     "sharpi_attention_latent": [P, P, I, P, P, P, P, P, I, I, F, I, I, I, I, I, I, I, P],
+    "sharpi_attention_latent_mfma": [P, P, P, P, P, P, P, I, I, P, P, P, P, F, I, I, I, I, I, I, I, I, P],
+    "sharpi_attention_latent_merge": [P, P, P, P, I, P, P, I, I, I, I, P],
     "sharpi_moe_permute": [P, P, P, P, P, P, P, I, I, I, I, I, P],
     "sharpi_gemm_grouped": [P, I, P, P, I, I, I, I, P, P, P, I, I, I, P],
     "sharpi_gemm_grouped_swiglu": [P, I, P, P, I, I, I, P, P, P, I, P, I, I, I, P],
@@ -124,6 +126,16 @@ def attention_takes(kind: str, hd: int) -> bool:
         fn = getattr(load(), f"sharpi_attention_{kind}_takes")
         fn.argtypes, fn.restype = [c_int], c_int
         _takes[key] = bool(fn(int(hd)))
+    return _takes[key]
+
+
+def latent_attention_takes(rank: int, dr: int) -> bool:
+    """Whether the matrix-core latent attention kernel takes a latent of `rank` and a rotated part of `dr` elements."""
+    key = ("latent", int(rank), int(dr))
+    if key not in _takes:
+        fn = load().sharpi_attention_latent_mfma_takes
+        fn.argtypes, fn.restype = [c_int, c_int], c_int
+        _takes[key] = bool(fn(int(rank), int(dr)))
     return _takes[key]
 
 

@@ -170,15 +170,26 @@ def test_products_per_head_and_the_gate(dtype, T, H, N, K):
 
 
 class _Ctx:
-    def __init__(self, entry_of, positions):
+    """What the attention op reads of a step: per-token arrays and the work lists (tokens of one
+    request: `tiles` cuts them into prompt tiles of tile_tokens, `singles` lists them one by one)."""
+
+    def __init__(self, entry_of, positions, tiles=False, singles=False, tile_tokens=64):
         self.entry_of_token, self.positions = entry_of, positions
         self.n_decode, self.decode_tokens, self.n_prefill_tiles, self.prefill_tiles = 0, None, 0, None
+        self.prefill_tile_tokens = tile_tokens
+        T = positions.shape[0]
+        if tiles:
+            t = [(0, o, min(tile_tokens, T - o)) for o in range(0, T, tile_tokens)]
+            self.prefill_tiles = torch.tensor(t, dtype=torch.int32, device=positions.device)
+            self.n_prefill_tiles = len(t)
+        if singles:
+            self.n_decode = T
 
 
 class _Group:
-    def __init__(self, bt):
+    def __init__(self, bt, max_context=0):
         self.block_table = bt
-        self.max_context = 0
+        self.max_context = max_context
 
 
 def _latent_case(H, R, dr, S, dtype, seed, far_key=None, sharpen=30.0):
@@ -224,27 +235,63 @@ def test_attention_over_latent_rows_with_a_sink(dtype, H, R, dr, S):
     ctx = _Ctx(torch.zeros(S, dtype=torch.int32, device=DEV), pos.to(DEV))
     scale = 1.0 / math.sqrt(R + dr)
     out = ops.attention_latent(q.reshape(S, -1).to(DEV), rows.to(DEV), _Group(bt.to(DEV)), ctx, scale, H, R, dr,
-                               sink=sink.to(DEV))
+                               sink=sink.to(DEV), kernel="generic")
     want = _plain_latent(q, keys, sink, scale, R, pos.long())
     assert _rel_rms(out.cpu().reshape(S, -1), want.reshape(S, -1)) < (2e-5 if dtype == "float32" else 8e-3)
-    none = ops.attention_latent(q.reshape(S, -1).to(DEV), rows.to(DEV), _Group(bt.to(DEV)), ctx, scale, H, R, dr)
+    none = ops.attention_latent(q.reshape(S, -1).to(DEV), rows.to(DEV), _Group(bt.to(DEV)), ctx, scale, H, R, dr, kernel="generic")
     want0 = _plain_latent(q, keys, torch.full((H,), -1e30), scale, R, pos.long())
     assert _rel_rms(none.cpu().reshape(S, -1), want0.reshape(S, -1)) < (2e-5 if dtype == "float32" else 8e-3)
     assert _rel_rms(out.cpu().reshape(S, -1), want0.reshape(S, -1)) > 0.05      # the sink is no small thing here
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("how", ["tiles", "singles"])
+@pytest.mark.parametrize("H, R, dr, S", [(3, 64, 16, 50), (5, 96, 16, 130), (8, 96, 16, 1100), (16, 128, 32, 77), (1, 16, 8, 40),
+                                         (20, 512, 64, 70), (40, 256, 32, 300), (70, 32, 0, 65)])
+def test_the_matrix_core_kernel_over_latent_rows(H, R, dr, S, how):
+    """Prompt tiles and listed single tokens through the matrix-core kernel: rows of several tokens in a
+    wave (few heads), several head tiles (many heads), one run and several (merged afterwards)."""
+    from sharpinference_amd import ops
+
+    q, keys, rows, bt = _latent_case(H, R, dr, S, "bfloat16", seed=S + H)
+    sink = torch.linspace(-4.0, 4.0, H) if H > 1 else torch.tensor([1.0])
+    pos = torch.arange(S, dtype=torch.int32)
+    scale = 1.0 / math.sqrt(R + dr)
+    want = _plain_latent(q, keys, sink, scale, R, pos.long())
+    ctx = _Ctx(torch.zeros(S, dtype=torch.int32, device=DEV), pos.to(DEV), tiles=how == "tiles", singles=how == "singles")
+    assert ops.latent_mfma_ok(torch.bfloat16, R, dr)
+    out = ops.attention_latent(q.reshape(S, -1).to(DEV), rows.to(DEV), _Group(bt.to(DEV), S), ctx, scale, H, R, dr,
+                               sink=sink.to(DEV), kernel="mfma")
+    assert _rel_rms(out.cpu().reshape(S, -1), want.reshape(S, -1)) < 8e-3
+    # the same rows through the float kernel, and without sinks
+    gen = ops.attention_latent(q.reshape(S, -1).to(DEV), rows.to(DEV), _Group(bt.to(DEV), S), ctx, scale, H, R, dr,
+                               sink=sink.to(DEV), kernel="generic")
+    assert _rel_rms(out.cpu().reshape(S, -1), gen.cpu().reshape(S, -1)) < 8e-3
+    none = ops.attention_latent(q.reshape(S, -1).to(DEV), rows.to(DEV), _Group(bt.to(DEV), S), ctx, scale, H, R, dr, kernel="mfma")
+    want0 = _plain_latent(q, keys, torch.full((H,), -1e30), scale, R, pos.long())
+    assert _rel_rms(none.cpu().reshape(S, -1), want0.reshape(S, -1)) < 8e-3
+
+
+def test_sizes_the_matrix_core_kernel_refuses_go_to_the_float_kernel():
+    from sharpinference_amd import ops
+
+    assert not ops.latent_mfma_ok(torch.bfloat16, 40, 8) and not ops.latent_mfma_ok(torch.float32, 64, 16)
+    assert not ops.latent_mfma_ok(torch.bfloat16, 64, 12) and not ops.latent_mfma_ok(torch.bfloat16, 512, 192)
+    assert ops.latent_run_keys(700, False) == ops.latent_run_keys(70000, False) == 256
+    assert [ops.latent_run_keys(n, True) for n in (5, 2048, 2049, 9000)] == [1024, 1024, 2048, 8192]
+
+
+@pytest.mark.parametrize("dtype, kernel", [("float32", "generic"), ("bfloat16", "generic"), ("bfloat16", "mfma")])
 @pytest.mark.parametrize("far_key", [0, 3, 15, 16, 17, 255, 256, 640, 689])
-def test_one_key_among_hundreds_is_found_wherever_it_lies(dtype, far_key):
+def test_one_key_among_hundreds_is_found_wherever_it_lies(dtype, kernel, far_key):
     from sharpinference_amd import ops
 
     H, R, dr, S = 4, 64, 16, 691
     q, keys, rows, bt = _latent_case(H, R, dr, S, dtype, seed=far_key, far_key=far_key)
     sink = torch.zeros(H)
     last = torch.tensor([S - 1], dtype=torch.int32)
-    ctx = _Ctx(torch.zeros(1, dtype=torch.int32, device=DEV), last.to(DEV))
-    out = ops.attention_latent(q[S - 1:].reshape(1, -1).to(DEV), rows.to(DEV), _Group(bt.to(DEV)), ctx, 1.0, H, R, dr,
-                               sink=sink.to(DEV))
+    ctx = _Ctx(torch.zeros(1, dtype=torch.int32, device=DEV), last.to(DEV), singles=True)
+    out = ops.attention_latent(q[S - 1:].reshape(1, -1).to(DEV), rows.to(DEV), _Group(bt.to(DEV), S), ctx, 1.0, H, R, dr,
+                               sink=sink.to(DEV), kernel=kernel)
     want = _plain_latent(q[S - 1:], keys, sink, 1.0, R, last.long())
     # the key that stands out carries the result: leaving it out (or taking its neighbour) is an error of order one
     assert _rel_rms(want.reshape(1, -1), keys[far_key, :R].double().repeat(H)[None]) < 0.05
