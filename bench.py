@@ -219,8 +219,8 @@ def decode_run(eng, batch: int, steps: int, warmup: int, rng: random.Random, cou
     return dt, distinct, ctx, host_ms
 
 
-def profile_report(eng, batch: int, prompt_len: int, rng: random.Random) -> None:
-    """ms / bytes / GB/s / TFLOP/s per kernel class of one prefill and one decode step (stderr)."""
+def profile_report(eng, batch: int, prompt_len: int, rng: random.Random):
+    """ms / bytes / GB/s / TFLOP/s per kernel class of one prefill and one decode step (stderr); returns the two tables."""
     from sharpinference_amd.engine import StepEntry
     from sharpinference_amd.ops.profile import Profiler, format_table
 
@@ -234,7 +234,8 @@ def profile_report(eng, batch: int, prompt_len: int, rng: random.Random) -> None
             eng.profiled_step(entry, prof)
         else:
             eng.step(entry)
-    log("\n" + format_table(prof.table(), f"prefill of one prompt of {prompt_len} tokens, by kernel class (event pairs):"))
+    pre_table = prof.table()
+    log("\n" + format_table(pre_table, f"prefill of one prompt of {prompt_len} tokens, by kernel class (event pairs):"))
     decode = [StepEntry(r, (rng.randrange(vocab),), (0,)) for r in ids]
     eng.step(decode, select="argmax")                       # warm
     prof = Profiler()
@@ -244,6 +245,7 @@ def profile_report(eng, batch: int, prompt_len: int, rng: random.Random) -> None
                                           "part behind filler work, by kernel class (event pairs):"))
     for r in ids:
         eng.free_request(r)
+    return pre_table, prof.table()
 
 
 def host_report(eng, prompt_len: int, rng: random.Random, batch: int = 64) -> dict:
@@ -457,6 +459,88 @@ def run_long16(args) -> int:
     return 0
 
 
+# ---------------------------------------------------------------------------
+# Kuvonex beside Llama 4 at equal sizes
+# ---------------------------------------------------------------------------
+# width, layers, heads, experts, picks, expert width, vocabulary; the latent layers take 128 + 64
+# wide query heads over a latent of 512, the Llama 4 layers heads of 128 in groups of 8 over a key head
+KUVONEX_SIZES = {
+    "w2048": dict(width=2048, layers=4, heads=16, experts=64, top=6, ff=1408, groups=(8, 4), vocab=32000),
+    "w4096": dict(width=4096, layers=2, heads=64, experts=32, top=4, ff=2048, groups=(4, 2), vocab=32000),
+}
+
+
+def kuvonex_config(z: dict) -> dict:
+    mixer = {"heads": z["heads"], "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "scale": 192 ** -0.5,
+             "rot": {"base": 10000.0, "dims": 64}}
+    mlp = {"kind": "moe", "expert": {"ff": z["ff"]},
+           "router": {"experts": z["experts"], "top": z["top"], "groups": {"count": z["groups"][0], "keep": z["groups"][1]}}}
+    layers = [{"type": "latent_attention", "mixer": dict(mixer), "mlp": mlp} for _ in range(z["layers"])]
+    layers[-1]["mixer"]["kv_from"] = z["layers"] - 2          # the last layer attends over its neighbour's latents
+    return {"architecture": "Kuvonex", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-5},
+            "embedding": {"scale": 1.0}, "layers": layers}
+
+
+def llama4_config_like(z: dict) -> dict:
+    cfg = dict(SCOUT)
+    cfg.update({"hidden_size": z["width"], "num_hidden_layers": z["layers"], "num_attention_heads": z["heads"],
+                "num_key_value_heads": max(1, z["heads"] // 8), "head_dim": 128, "vocab_size": z["vocab"],
+                "intermediate_size": z["ff"], "intermediate_size_mlp": z["ff"], "num_local_experts": z["experts"],
+                "num_experts_per_tok": z["top"], "interleave_moe_layer_step": 1, "rope_scaling": None,
+                "no_rope_layers": [0 if (l + 1) % 4 == 0 else 1 for l in range(z["layers"])], "max_position_embeddings": CONTEXT})
+    return cfg
+
+
+def run_kuvonex(args) -> int:
+    """Prefill of one 2,048-token prompt and decode at batch 8 and 64 for the Kuvonex design at two
+    sizes, each beside Llama 4 layers of the same width, heads, experts and expert width (random
+    weights), with the per-kernel-class tables of one prefill and one decode step of both."""
+    import torch
+    from sharpinference_amd.engine import Engine
+
+    P, steps, warm = args.prompt_len, min(args.steps, 48), 4
+    per_req = (P + steps + warm + 16 + args.page_size - 1) // args.page_size * args.page_size + 2 * args.page_size
+    rows = []
+    for size, z in KUVONEX_SIZES.items():
+        for model, cfg in (("kuvonex", kuvonex_config(z)), ("llama4", llama4_config_like(z))):
+            t0 = time.time()
+            eng = Engine(config=cfg, weight_seed=2, dtype="bfloat16", device="cuda:0", max_model_len=CONTEXT, max_num_seqs=64,
+                         max_tokens_per_step=8192, kv_tokens=64 * per_req, page_size=args.page_size,
+                         decode_graphs=not args.no_graphs)
+            log(f"{model} {size}: engine ready in {time.time() - t0:.1f}s")
+            rng = random.Random(5)
+            prompt = [rng.randrange(z["vocab"]) for _ in range(P)]
+            best = None
+            for i in range(4):                                  # once to warm up, then three times timed
+                dt, _ = run_prefill(eng, f"pre{i}", prompt)
+                eng.free_request(f"pre{i}")
+                best = dt if i and (best is None or dt < best) else best
+            row = {"size": size, "model": model, "prefill_tok_s": P / best, "prefill_ms": best * 1e3}
+            for batch in (8, 64):
+                dt, _, ctx, host_ms = decode_run(eng, batch, steps, warm, rng, prompt_len=P)
+                row[f"decode_b{batch}_tok_s"] = batch * steps / dt
+                row[f"decode_b{batch}_ms_per_step"] = dt / steps * 1e3
+            log(f"{model} {size}: prefill {row['prefill_ms']:.2f} ms ({row['prefill_tok_s']:.0f} tok/s), decode b8 "
+                f"{row['decode_b8_ms_per_step']:.3f} ms/step, b64 {row['decode_b64_ms_per_step']:.3f} ms/step")
+            pre, dec = profile_report(eng, 8, P, rng)
+            row["prefill_classes"] = {k: {"ms": round(v["ms"], 4), "gbs": round(v["bytes"] / v["ms"] / 1e6, 1) if v["ms"] else 0,
+                                          "tflops": round(v["flops"] / v["ms"] / 1e9, 2) if v["ms"] else 0} for k, v in pre.items()}
+            row["decode_b8_classes"] = {k: {"ms": round(v["ms"], 4), "gbs": round(v["bytes"] / v["ms"] / 1e6, 1) if v["ms"] else 0}
+                                        for k, v in dec.items()}
+            rows.append(row)
+            del eng
+            torch.cuda.empty_cache()
+    k0 = rows[0]
+    out = {"metric": "decode tok/s at batch 8 (Kuvonex, width 2048, 4 layers, 2,048-token prompts)", "value": k0["decode_b8_tok_s"],
+           "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": k0["decode_b8_ms_per_step"],
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+           "config": {"model": "kuvonex-random beside llama4-random at equal sizes", "global_batch": 8, "seq_len": CONTEXT,
+                      "parallelism": "single-gpu", "prompt_len": P, "sizes": KUVONEX_SIZES},
+           "rows": rows}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -470,8 +554,9 @@ def main() -> int:
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel instead of replaying a HIP graph")
     ap.add_argument("--no-peaks", action="store_true", help="skip the two measuring kernels (pure read, matrix-core loop)")
     ap.add_argument("--profile", action="store_true", help="also print ms / bytes / GB/s per kernel class of one prefill and one decode step")
-    ap.add_argument("--shape", default="scout", choices=["scout", "maverick8", "long16"],
-                    help="scout: the headline run; maverick8 / long16: two other workloads, each printing a JSON line of its own")
+    ap.add_argument("--shape", default="scout", choices=["scout", "maverick8", "long16", "kuvonex"],
+                    help="scout: the headline run; maverick8 / long16: two other workloads; kuvonex: the Kuvonex design beside "
+                         "Llama 4 layers of equal size; each prints a JSON line of its own")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this engine has no multi-GPU path (N=1 only)")
@@ -480,6 +565,8 @@ def main() -> int:
         return run_maverick8(args)
     if args.shape == "long16":
         return run_long16(args)
+    if args.shape == "kuvonex":
+        return run_kuvonex(args)
 
     import torch  # noqa: F401
 

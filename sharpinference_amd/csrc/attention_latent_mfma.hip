@@ -2,9 +2,12 @@
 // [c (R) | rotated key part (dr)], score = q . row over D = R + dr elements, value = the row's
 // first R elements.
 //
-// A block of four waves works on up to 64 (token, head) rows of one request against one run of
-// keys [run * RUN, (run + 1) * RUN): a wave owns 16 rows (16 heads of a token, or all heads of
-// several consecutive tokens where a layer has fewer than 16) and every output element of them.
+// A block of eight waves works on up to 64 (token, head) rows of one request against one run of
+// keys [run * RUN, (run + 1) * RUN): 16 rows (16 heads of a token, or all heads of several
+// consecutive tokens where a layer has fewer than 16) belong to a pair of waves, each of which
+// forms the scores and the softmax state of the rows (the same bits in both) and one half of their
+// output elements, so that a wave's accumulators take 64 registers for a latent of 512 and two
+// waves fit a SIMD.
 // Keys come in chunks of 32, staged in LDS once for the block: the rows as they lie in the cache
 // (the A operand of S^T = K Q^T, contraction over elements), and their first R elements once more,
 // transposed [element][key] (the A operand of O^T = V^T P^T, contraction over keys), made from the
@@ -19,7 +22,8 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-constexpr int kLmWaves = 4;
+constexpr int kLmWaves = 4;           // row groups of 16 rows a block
+constexpr int kLmHalves = 2;          // waves a row group: each takes half of the output elements
 constexpr int kLmChunk = 32;          // keys a chunk
 constexpr int kLmVtLd = kLmChunk + 8; // elements a row of the transposed tile (rows 16 bytes apart in banks)
 
@@ -35,7 +39,7 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
 }
 
 template <int MAXD32, int MAXR16>
-__global__ __launch_bounds__(kLmWaves* kWave) void attn_latent_mfma_kernel(
+__global__ __launch_bounds__(kLmWaves* kLmHalves* kWave) void attn_latent_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ rows, const int* __restrict__ block_table,
     const int* __restrict__ entry_of_token, const int* __restrict__ positions, const int* __restrict__ tiles,
     const int* __restrict__ token_list, int tile_subs, const float* __restrict__ sink, bf16_t* __restrict__ out,
@@ -46,9 +50,13 @@ __global__ __launch_bounds__(kLmWaves* kWave) void attn_latent_mfma_kernel(
   bf16_t* vt = kt + kLmChunk * gm.ldk;                             // [R][kLmVtLd], keys in the order the second product wants
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
-  const int w = tid >> 6;
+  const int w = (tid >> 6) & (kLmWaves - 1), half = tid >> 8;
   const int g = lane >> 4, m16 = lane & 15;
   const int tpb = gm.tgb * gm.tb;
+  // this wave's 16-element tiles of the output: the first or the second half of them
+  constexpr int MAXH = (MAXR16 + 1) / 2;
+  const int r_lo = half ? (gm.r16 + 1) / 2 : 0;
+  const int r_n = half ? gm.r16 - r_lo : (gm.r16 + 1) / 2;
 
   // the block's tokens: a piece of a prompt tile, or one listed token
   int tok0, cnt, e;
@@ -93,27 +101,49 @@ __global__ __launch_bounds__(kLmWaves* kWave) void attn_latent_mfma_kernel(
   // the columns of the staged rows beyond D stay zero
   for (int i = tid; i < kLmChunk * gm.ldk / 8; i += blockDim.x) reinterpret_cast<uint4*>(kt)[i] = make_uint4(0, 0, 0, 0);
 
-  f32x4 acc[MAXR16];
+  f32x4 acc[MAXH];
 #pragma unroll
-  for (int d = 0; d < MAXR16; ++d) acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int d = 0; d < MAXH; ++d) acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
   const int d8 = gm.D >> 3;
-  const int n_pieces = kLmChunk * d8;
+  // Staging: a thread owns row (tid / 16) of every chunk and the pieces of 8 elements c, c + 16, ... of
+  // it (sixteen lanes read 256 bytes on end), so a chunk costs it ONE page lookup, which is made a
+  // chunk ahead, and NJ independent loads, which are requested before the chunk before is multiplied.
+  constexpr int NJ = (MAXD32 * 4 + 15) / 16;
+  const int st_r = tid >> 4, st_c = tid & 15;
+  auto row_of = [&](int c0) -> const bf16_t* {
+    const int key = c0 + st_r;
+    if (key >= k_end) return nullptr;
+    const int blk = key / page_size;
+    const int page = blk < max_blocks ? bt[blk] : -1;
+    return (page >= 0 && page < num_pages) ? rows + ((size_t)page * page_size + key % page_size) * gm.D : nullptr;
+  };
+  uint4 stage[NJ];
+  auto fetch = [&](const bf16_t* src) {
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int c8 = st_c + 16 * j;
+      stage[j] = (src && c8 < d8) ? *reinterpret_cast<const uint4*>(src + 8 * c8) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  // (with the widest rows the registers do not reach for rows held across the products: they are
+  // then requested where they are stored, and the SIMD's other wave covers the wait)
+  constexpr bool kAhead = MAXD32 <= 10;
+  const bf16_t* cur_row = row_of(k_begin);
+  if (kAhead) fetch(cur_row);
+  const bf16_t* next_row = row_of(k_begin + kLmChunk);
 
   for (int c0 = k_begin; c0 < k_end; c0 += kLmChunk) {
+    if (!kAhead) fetch(cur_row);
     __syncthreads();                       // the chunk before is used up (the first time: the zero fill is done)
-    for (int piece = tid; piece < n_pieces; piece += blockDim.x) {
-      const int r = piece / d8, c8 = piece - r * d8;
-      const int key = c0 + r;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (key < k_end) {
-        const int blk = key / page_size;
-        const int page = blk < max_blocks ? bt[blk] : -1;
-        if (page >= 0 && page < num_pages)
-          v = *reinterpret_cast<const uint4*>(rows + ((size_t)page * page_size + key % page_size) * gm.D + 8 * c8);
-      }
-      *reinterpret_cast<uint4*>(kt + r * gm.ldk + 8 * c8) = v;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int c8 = st_c + 16 * j;
+      if (c8 < d8) *reinterpret_cast<uint4*>(kt + st_r * gm.ldk + 8 * c8) = stage[j];
     }
+    if (kAhead) fetch(next_row);           // the next chunk's rows are on their way while this one is transposed and multiplied
+    cur_row = next_row;
+    next_row = row_of(c0 + 2 * kLmChunk);
     __syncthreads();
     // element d of keys {4 gq + i, 16 + 4 gq + i} -> vt[d][8 gq ..]: the order in which a lane of the
     // first product holds its probabilities
@@ -176,13 +206,17 @@ __global__ __launch_bounds__(kLmWaves* kWave) void attn_latent_mfma_kernel(
       lo = make_uint4(pack_bf16(r[0], r[1]), pack_bf16(r[2], r[3]), pack_bf16(r[4], r[5]), pack_bf16(r[6], r[7]));
     }
     const bf16x8 pf_hi = *reinterpret_cast<bf16x8*>(&hi), pf_lo = *reinterpret_cast<bf16x8*>(&lo);
+    if (__any(corr != 1.0f)) {             // some row's maximum moved: seldom, once the first chunks are through
 #pragma unroll
-    for (int d = 0; d < MAXR16; ++d) {
-      if (d < gm.r16) {
-        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vt + (16 * d + m16) * kLmVtLd + 8 * g);
-        f32x4 a = acc[d];
-        a[0] *= corr; a[1] *= corr; a[2] *= corr; a[3] *= corr;
-        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf_hi, a, 0, 0, 0);
+      for (int d = 0; d < MAXH; ++d) {
+        acc[d][0] *= corr; acc[d][1] *= corr; acc[d][2] *= corr; acc[d][3] *= corr;
+      }
+    }
+#pragma unroll
+    for (int d = 0; d < MAXH; ++d) {
+      if (d < r_n) {
+        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vt + (16 * (r_lo + d) + m16) * kLmVtLd + 8 * g);
+        const f32x4 a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf_hi, acc[d], 0, 0, 0);
         acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf_lo, a, 0, 0, 0);
       }
     }
@@ -200,10 +234,10 @@ __global__ __launch_bounds__(kLmWaves* kWave) void attn_latent_mfma_kernel(
       denom = l_run * expf(m_run - M) + expf(sk - M);
     }
     const float f = denom > 0.f ? expf(m_run - M) / denom : 0.f;
-    bf16_t* orow = out + rh * gm.R;
+    bf16_t* orow = out + rh * gm.R + 16 * r_lo;
 #pragma unroll
-    for (int d = 0; d < MAXR16; ++d) {
-      if (d < gm.r16) {
+    for (int d = 0; d < MAXH; ++d) {
+      if (d < r_n) {
         uint2 v;
         v.x = pack_bf16(acc[d][0] * f, acc[d][1] * f);
         v.y = pack_bf16(acc[d][2] * f, acc[d][3] * f);
@@ -212,45 +246,59 @@ __global__ __launch_bounds__(kLmWaves* kWave) void attn_latent_mfma_kernel(
     }
     return;
   }
-  float* po = part_o + (rh * max_runs + run) * gm.R;
+  float* po = part_o + (rh * max_runs + run) * gm.R + 16 * r_lo;
 #pragma unroll
-  for (int d = 0; d < MAXR16; ++d) {
-    if (d < gm.r16) *reinterpret_cast<float4*>(po + 16 * d + 4 * g) = make_float4(acc[d][0], acc[d][1], acc[d][2], acc[d][3]);
+  for (int d = 0; d < MAXH; ++d) {
+    if (d < r_n) *reinterpret_cast<float4*>(po + 16 * d + 4 * g) = make_float4(acc[d][0], acc[d][1], acc[d][2], acc[d][3]);
   }
-  if (g == 0) {
+  if (g == 0 && half == 0) {
     part_ml[(rh * max_runs + run) * 2] = m_run;
     part_ml[(rh * max_runs + run) * 2 + 1] = l_run;
   }
 }
 
-// One block per (token, head) with more than one run: out = sum_r o_r e^(m_r - M) / (sum_r l_r e^(m_r - M) + e^(sink - M)).
-__global__ __launch_bounds__(128) void attn_latent_merge_kernel(const float* __restrict__ part_o,
-                                                                const float* __restrict__ part_ml,
-                                                                const int* __restrict__ positions,
-                                                                const int* __restrict__ token_list,
-                                                                const float* __restrict__ sink,
-                                                                bf16_t* __restrict__ out, int H, int R, int run_keys,
-                                                                int max_runs) {
+// The rows with more than one run: out = sum_r o_r e^(m_r - M) / (sum_r l_r e^(m_r - M) + e^(sink - M)), a wave a
+// (token, head) row, four rows a block.  The maximum and the denominator are taken with a lane a run
+// (wave reductions in a fixed order), the output with a lane per four elements, runs in ascending order.
+constexpr int kLmMergeWaves = 4;
+
+__global__ __launch_bounds__(kLmMergeWaves* kWave) void attn_latent_merge_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ positions,
+    const int* __restrict__ token_list, const float* __restrict__ sink, bf16_t* __restrict__ out, int H, int R,
+    int run_keys, int max_runs) {
   const int token = token_list ? token_list[blockIdx.x] : blockIdx.x;
-  const int head = blockIdx.y;
+  const int head = blockIdx.y * kLmMergeWaves + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & (kWave - 1);
+  if (head >= H) return;
   const int n_runs = positions[token] / run_keys + 1;
   if (n_runs <= 1) return;
   const size_t rh = (size_t)token * H + head;
   bf16_t* orow = out + rh * R;
   if (n_runs > max_runs) {          // the launch was sized for fewer keys than this token sees: never a result over fewer keys
-    for (int d = threadIdx.x; d < R; d += blockDim.x) orow[d].bits = 0x7fc0;
+    for (int d = lane; d < R; d += kWave) orow[d].bits = 0x7fc0;
     return;
   }
   const float* ml = part_ml + rh * max_runs * 2;
-  float M = sink ? sink[head] : -INFINITY;
-  for (int r = 0; r < n_runs; ++r) M = fmaxf(M, ml[2 * r]);
-  float denom = sink ? expf(sink[head] - M) : 0.f;
-  for (int r = 0; r < n_runs; ++r) denom += ml[2 * r + 1] * expf(ml[2 * r] - M);
+  float mx = -INFINITY;
+  for (int r = lane; r < n_runs; r += kWave) mx = fmaxf(mx, ml[2 * r]);
+  float M = wave_max(mx);
+  if (sink) M = fmaxf(M, sink[head]);
+  float dl = 0.f;
+  for (int r = lane; r < n_runs; r += kWave) dl += ml[2 * r + 1] * expf(ml[2 * r] - M);
+  const float denom = wave_sum(dl) + (sink ? expf(sink[head] - M) : 0.f);
   const float inv = denom > 0.f ? 1.0f / denom : 0.f;
-  for (int d = threadIdx.x; d < R; d += blockDim.x) {
-    float o = 0.f;
-    for (int r = 0; r < n_runs; ++r) o += part_o[(rh * max_runs + r) * R + d] * expf(ml[2 * r] - M);
-    orow[d] = f32_to_bf16(o * inv);
+  const float* po = part_o + rh * max_runs * R;
+  for (int d = 4 * lane; d < R; d += 4 * kWave) {
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int r = 0; r < n_runs; ++r) {
+      const float wr = expf(ml[2 * r] - M);
+      const float4 v = *reinterpret_cast<const float4*>(po + (size_t)r * R + d);
+      o.x += v.x * wr; o.y += v.y * wr; o.z += v.z * wr; o.w += v.w * wr;
+    }
+    uint2 pk;
+    pk.x = pack_bf16(o.x * inv, o.y * inv);
+    pk.y = pack_bf16(o.z * inv, o.w * inv);
+    *reinterpret_cast<uint2*>(orow + d) = pk;
   }
 }
 
@@ -305,7 +353,7 @@ SHARPI_EXPORT int sharpi_attention_latent_mfma(const void* q, const void* rows, 
   const int subs = tiles ? ceil_div(tile_tokens, tpb) : 1;
   const int head_blocks = ceil_div(ceil_div(H, g.hpw), g.htb);
   if (head_blocks > 65535) return SHARPI_ERR_ARG;
-  dim3 grid(n_items * subs, max_runs, head_blocks), block(kLmWaves * kWave);
+  dim3 grid(n_items * subs, max_runs, head_blocks), block(kLmWaves * kLmHalves * kWave);
   const size_t lds = ((size_t)kLmChunk * g.ldk + (size_t)R * kLmVtLd) * sizeof(bf16_t);
 #define LM_LAUNCH(MD, MR)                                                                                         \
   do {                                                                                                            \
@@ -331,8 +379,8 @@ SHARPI_EXPORT int sharpi_attention_latent_merge(const float* part_o, const float
                                                 const int* token_list, int n_tokens, const float* sink, void* out,
                                                 int H, int R, int run_keys, int max_runs, hipStream_t stream) {
   if (n_tokens <= 0 || max_runs <= 1) return SHARPI_OK;
-  if (H <= 0 || H > 65535 || R <= 0 || run_keys <= 0) return SHARPI_ERR_ARG;
-  dim3 grid(n_tokens, H), block(128);
+  if (H <= 0 || H > 65535 || R <= 0 || R % 4 || run_keys <= 0) return SHARPI_ERR_ARG;
+  dim3 grid(n_tokens, ceil_div(H, kLmMergeWaves)), block(kLmMergeWaves * kWave);
   attn_latent_merge_kernel<<<grid, block, 0, stream>>>(part_o, part_ml, positions, token_list, sink, (bf16_t*)out, H, R,
                                                        run_keys, max_runs);
   SHARPI_CHECK_LAUNCH();

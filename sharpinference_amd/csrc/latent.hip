@@ -211,6 +211,73 @@ __global__ __launch_bounds__(256) void head_gemm_kernel(const T* __restrict__ x,
   }
 }
 
+// The same on the matrix cores (bfloat16): a block of four waves computes 64 tokens x 64 outputs of
+// one head, a wave 32 x 32 as 2 x 2 tiles of v_mfma_f32_16x16x32_bf16 with the weights as the A
+// operand (out^T = W x^T); both operands come straight from memory in runs of 8 elements (a head's
+// weights are small and stay in cache).  Every output is one chain over k in the same order whatever
+// the number of tokens.  K, the heads' input stride and the row strides are multiples of 8 elements,
+// the output's of 4.
+typedef __attribute__((ext_vector_type(8))) __bf16 hg_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float hg_f32x4;
+
+__global__ __launch_bounds__(256) void head_gemm_mfma_kernel(const bf16_t* __restrict__ x, int ldx, int sx,
+                                                             const bf16_t* __restrict__ w, bf16_t* __restrict__ out,
+                                                             int ldo, int so, const bf16_t* __restrict__ gate, int ldg,
+                                                             int n_tokens, int N, int K) {
+  const int h = blockIdx.z;
+  const int wv = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
+  const int g = lane >> 4, m = lane & 15;
+  const int t_base = blockIdx.x * 64 + (wv >> 1) * 32, n_base = blockIdx.y * 64 + (wv & 1) * 32;
+  if (t_base >= n_tokens || n_base >= N) return;
+  const bf16_t* xp[2];
+  const bf16_t* wp[2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+    xp[a] = x + (size_t)min(t_base + 16 * a + m, n_tokens - 1) * ldx + (size_t)h * sx + 8 * g;
+    wp[a] = w + ((size_t)h * N + min(n_base + 16 * a + m, N - 1)) * K + 8 * g;
+  }
+  hg_f32x4 acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) acc[a][b] = hg_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const bool in = k0 + 8 * g < K;
+    uint4 xa[2], wa[2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      xa[a] = in ? *reinterpret_cast<const uint4*>(xp[a] + k0) : make_uint4(0, 0, 0, 0);
+      wa[a] = in ? *reinterpret_cast<const uint4*>(wp[a] + k0) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<hg_bf16x8*>(&wa[a]),
+                                                            *reinterpret_cast<hg_bf16x8*>(&xa[b]), acc[a][b], 0, 0, 0);
+  }
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    const int t = t_base + 16 * b + m;
+    if (t >= n_tokens) continue;
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      const int n = n_base + 16 * a + 4 * g;
+      if (n >= N) continue;                       // (N is a multiple of 4: the four outputs are in or out together)
+      float v[4] = {acc[a][b][0], acc[a][b][1], acc[a][b][2], acc[a][b][3]};
+      if (gate) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] *= 1.0f / (1.0f + expf(-bf16_to_f32(gate[(size_t)t * ldg + (size_t)h * N + n + i])));
+      }
+      uint2 o;
+      o.x = (uint32_t)f32_to_bf16(v[0]).bits | ((uint32_t)f32_to_bf16(v[1]).bits << 16);
+      o.y = (uint32_t)f32_to_bf16(v[2]).bits | ((uint32_t)f32_to_bf16(v[3]).bits << 16);
+      *reinterpret_cast<uint2*>(out + (size_t)t * ldo + (size_t)h * so + n) = o;
+    }
+  }
+}
+
 // x rows of ldx elements, head h's K inputs at column h * sx; w [H, N, K]; out rows of ldo elements,
 // head h's N outputs at column h * so; gate (or null) rows of ldg elements, head h's at column h * N:
 // the result is multiplied by sigmoid(gate).  All of one storage type.
@@ -225,6 +292,10 @@ SHARPI_EXPORT int sharpi_head_gemm(const void* x, int dtype, int ldx, int sx, co
   if (dtype == DT_F32)
     head_gemm_kernel<float><<<grid, block, 0, stream>>>((const float*)x, ldx, sx, (const float*)w, (float*)out, ldo, so,
                                                         (const float*)gate, ldg, n_tokens, N, K);
+  else if (dtype == DT_BF16 && K % 8 == 0 && sx % 8 == 0 && ldx % 8 == 0 && N % 4 == 0 && so % 4 == 0 && ldo % 4 == 0 &&
+           ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)out & 7) == 0)
+    head_gemm_mfma_kernel<<<grid, block, 0, stream>>>((const bf16_t*)x, ldx, sx, (const bf16_t*)w, (bf16_t*)out, ldo, so,
+                                                      (const bf16_t*)gate, ldg, n_tokens, N, K);
   else if (dtype == DT_BF16)
     head_gemm_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, ldx, sx, (const bf16_t*)w, (bf16_t*)out, ldo,
                                                          so, (const bf16_t*)gate, ldg, n_tokens, N, K);

@@ -474,7 +474,7 @@ def head_gemm(x: torch.Tensor, x_off: int, sx: int, w: torch.Tensor, out: torch.
 LATENT_MAX_RANK = 512    # the latent attention kernels hold this many value elements a row
 
 
-LATENT_DECODE_RUN_KEYS = 256     # keys a block of the matrix-core latent kernel walks in steps of single tokens
+LATENT_DECODE_RUN_KEYS = 128     # keys a block of the matrix-core latent kernel walks in steps of single tokens
 LATENT_PROMPT_RUN_KEYS = 1024    # ... at least, in steps with prompt portions (at most two runs a row)
 
 

@@ -148,24 +148,29 @@ def test_latent_rows_and_rotated_query_parts(dtype, H, dn, dr, R, dims):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("T, H, N, K", [(1, 3, 40, 24), (70, 5, 12, 40), (130, 2, 64, 64)])
-def test_products_per_head_and_the_gate(dtype, T, H, N, K):
+@pytest.mark.parametrize("xo, oo, pad", [(5, 2, 3), (8, 4, 4)])     # unaligned: the float kernel; aligned: the matrix cores in bfloat16
+@pytest.mark.parametrize("T, H, N, K", [(1, 3, 40, 24), (70, 5, 12, 40), (130, 2, 64, 64), (33, 4, 100, 136), (17, 1, 4, 8)])
+def test_products_per_head_and_the_gate(dtype, T, H, N, K, xo, oo, pad):
     from sharpinference_amd import ops
 
     g = torch.Generator().manual_seed(T)
-    sx, so = K + 8, N + 3
-    x = torch.randn(T, 5 + H * sx, generator=g).to(DT[dtype])
+    sx, so = K + 8, N + pad + 1 if pad == 3 else N + pad
+    x = torch.randn(T, xo + H * sx + (3 if pad == 3 else 0), generator=g).to(DT[dtype])
     w = (torch.randn(H, N, K, generator=g) * 0.3).to(DT[dtype])
     gate = torch.randn(T, 9 + H * N, generator=g).to(DT[dtype])
-    out = torch.zeros(T, 2 + H * so, dtype=DT[dtype], device=DEV)
-    ops.head_gemm(x.to(DEV), 5, sx, w.to(DEV), out, 2, so, gate=gate.to(DEV), gate_off=9)
-    xs = torch.stack([x.double()[:, 5 + h * sx: 5 + h * sx + K] for h in range(H)], 1)          # [T, H, K]
+    out = torch.zeros(T, oo + H * so + (1 if pad == 3 else 0), dtype=DT[dtype], device=DEV)
+    ops.head_gemm(x.to(DEV), xo, sx, w.to(DEV), out, oo, so, gate=gate.to(DEV), gate_off=9)
+    xs = torch.stack([x.double()[:, xo + h * sx: xo + h * sx + K] for h in range(H)], 1)          # [T, H, K]
     want = torch.einsum("thk,hnk->thn", xs, w.double()) * torch.sigmoid(gate.double()[:, 9:].reshape(T, H, N))
-    got = torch.stack([out.cpu().double()[:, 2 + h * so: 2 + h * so + N] for h in range(H)], 1)
+    got = torch.stack([out.cpu().double()[:, oo + h * so: oo + h * so + N] for h in range(H)], 1)
     assert _rel_rms(got.reshape(T, -1), want.reshape(T, -1)) < (1e-6 if dtype == "float32" else 4e-3)
+    untouched = torch.ones(out.shape[1], dtype=torch.bool)
+    for h in range(H):
+        untouched[oo + h * so: oo + h * so + N] = False
+    assert bool((out.cpu()[:, untouched] == 0).all())                 # nothing is written between the heads' outputs
     plain = torch.zeros_like(out)
-    ops.head_gemm(x.to(DEV), 5, sx, w.to(DEV), plain, 2, so)
-    got = torch.stack([plain.cpu().double()[:, 2 + h * so: 2 + h * so + N] for h in range(H)], 1)
+    ops.head_gemm(x.to(DEV), xo, sx, w.to(DEV), plain, oo, so)
+    got = torch.stack([plain.cpu().double()[:, oo + h * so: oo + h * so + N] for h in range(H)], 1)
     assert _rel_rms(got.reshape(T, -1), torch.einsum("thk,hnk->thn", xs, w.double()).reshape(T, -1)) < (1e-6 if dtype == "float32" else 4e-3)
 
 
@@ -276,7 +281,7 @@ def test_sizes_the_matrix_core_kernel_refuses_go_to_the_float_kernel():
 
     assert not ops.latent_mfma_ok(torch.bfloat16, 40, 8) and not ops.latent_mfma_ok(torch.float32, 64, 16)
     assert not ops.latent_mfma_ok(torch.bfloat16, 64, 12) and not ops.latent_mfma_ok(torch.bfloat16, 512, 192)
-    assert ops.latent_run_keys(700, False) == ops.latent_run_keys(70000, False) == 256
+    assert ops.latent_run_keys(700, False) == ops.latent_run_keys(70000, False) == ops.LATENT_DECODE_RUN_KEYS
     assert [ops.latent_run_keys(n, True) for n in (5, 2048, 2049, 9000)] == [1024, 1024, 2048, 8192]
 
 
