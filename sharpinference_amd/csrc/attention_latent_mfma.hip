@@ -358,9 +358,11 @@ SHARPI_EXPORT int sharpi_attention_latent_mfma(const void* q, const void* rows, 
 #define LM_LAUNCH(MD, MR)                                                                                         \
   do {                                                                                                            \
     auto kern = attn_latent_mfma_kernel<MD, MR>;                                                                  \
-    if (lds > 48 * 1024) {                                                                                        \
+    static size_t allowed = 48 * 1024;       /* dynamic LDS this instantiation may take (raised once per size) */  \
+    if (lds > allowed) {                                                                                          \
       hipError_t e_ = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
       if (e_ != hipSuccess) return (int)e_;                                                                       \
+      allowed = lds;                                                                                              \
     }                                                                                                             \
     kern<<<grid, block, lds, stream>>>((const bf16_t*)q, (const bf16_t*)rows, block_table, entry_of_token,        \
                                        positions, tiles, token_list, subs, sink, (bf16_t*)out, part_o, part_ml,   \

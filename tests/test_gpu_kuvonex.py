@@ -285,8 +285,26 @@ def test_sizes_the_matrix_core_kernel_refuses_go_to_the_float_kernel():
     assert [ops.latent_run_keys(n, True) for n in (5, 2048, 2049, 9000)] == [1024, 1024, 2048, 8192]
 
 
+@pytest.mark.parametrize("far_key", [0, 15, 16, 17, 1023, 1024, 1025, 1097])
+def test_one_key_among_a_thousand_is_found_in_a_prompt_tile(far_key):
+    """The same through prompt tiles of the matrix-core kernel: 1,099 positions query at once, the
+    last one looks for the key; keys on both sides of the 1,024-key run border and of page borders."""
+    from sharpinference_amd import ops
+
+    H, R, dr, S = 4, 64, 16, 1099
+    q, keys, rows, bt = _latent_case(H, R, dr, S, "bfloat16", seed=far_key, far_key=far_key)
+    sink = torch.zeros(H)
+    pos = torch.arange(S, dtype=torch.int32)
+    ctx = _Ctx(torch.zeros(S, dtype=torch.int32, device=DEV), pos.to(DEV), tiles=True)
+    out = ops.attention_latent(q.reshape(S, -1).to(DEV), rows.to(DEV), _Group(bt.to(DEV), S), ctx, 1.0, H, R, dr,
+                               sink=sink.to(DEV), kernel="mfma")
+    want = _plain_latent(q[S - 1:], keys, sink, 1.0, R, pos[S - 1:].long())
+    assert _rel_rms(want.reshape(1, -1), keys[far_key, :R].double().repeat(H)[None]) < 0.05
+    assert _rel_rms(out.cpu()[S - 1:].reshape(1, -1), want.reshape(1, -1)) < 1e-2
+
+
 @pytest.mark.parametrize("dtype, kernel", [("float32", "generic"), ("bfloat16", "generic"), ("bfloat16", "mfma")])
-@pytest.mark.parametrize("far_key", [0, 3, 15, 16, 17, 255, 256, 640, 689])
+@pytest.mark.parametrize("far_key", [0, 3, 15, 16, 17, 127, 128, 129, 255, 256, 640, 689])
 def test_one_key_among_hundreds_is_found_wherever_it_lies(dtype, kernel, far_key):
     from sharpinference_amd import ops
 

@@ -39,7 +39,7 @@ EVEN = {
     "layers": [
         _layer(_mixer(4, 32, 32, 32, 64, 0.125, 10000.0), _moe(8, 2, 128, (8, 4))),
         _layer(_mixer(8, 16, 32, 16, 64, 0.2, 10000.0, kv_from=0), _moe(8, 8, 128)),
-        _layer(_mixer(16, 64, 16, 64, 128, 0.09, 10000.0), _moe(4, 2, 256, (2, 2))),
+        _layer(_mixer(16, 64, 16, 64, 128, 0.09, 10000.0, dims=8), _moe(4, 2, 256, (2, 2))),   # half of the rotated part turns
     ],
 }
 
