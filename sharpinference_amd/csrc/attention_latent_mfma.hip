@@ -287,18 +287,25 @@ __global__ __launch_bounds__(kLmMergeWaves* kWave) void attn_latent_merge_kernel
   for (int r = lane; r < n_runs; r += kWave) dl += ml[2 * r + 1] * expf(ml[2 * r] - M);
   const float denom = wave_sum(dl) + (sink ? expf(sink[head] - M) : 0.f);
   const float inv = denom > 0.f ? 1.0f / denom : 0.f;
+  const float w_lane = lane < n_runs ? expf(ml[2 * lane] - M) : 0.f;     // run r's weight sits in lane r (the first 64 runs)
   const float* po = part_o + rh * max_runs * R;
-  for (int d = 4 * lane; d < R; d += 4 * kWave) {
+  for (int d0 = 0; d0 < R; d0 += 4 * kWave) {      // (every lane walks the loop: the weights come from other lanes)
+    const int d = d0 + 4 * lane;
+    const bool on = d < R;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int r = 0; r < n_runs; ++r) {
-      const float wr = expf(ml[2 * r] - M);
-      const float4 v = *reinterpret_cast<const float4*>(po + (size_t)r * R + d);
-      o.x += v.x * wr; o.y += v.y * wr; o.z += v.z * wr; o.w += v.w * wr;
+      const float wr = r < kWave ? __shfl(w_lane, r, kWave) : expf(ml[2 * r] - M);
+      if (on) {
+        const float4 v = *reinterpret_cast<const float4*>(po + (size_t)r * R + d);
+        o.x += v.x * wr; o.y += v.y * wr; o.z += v.z * wr; o.w += v.w * wr;
+      }
     }
-    uint2 pk;
-    pk.x = pack_bf16(o.x * inv, o.y * inv);
-    pk.y = pack_bf16(o.z * inv, o.w * inv);
-    *reinterpret_cast<uint2*>(orow + d) = pk;
+    if (on) {
+      uint2 pk;
+      pk.x = pack_bf16(o.x * inv, o.y * inv);
+      pk.y = pack_bf16(o.z * inv, o.w * inv);
+      *reinterpret_cast<uint2*>(orow + d) = pk;
+    }
   }
 }
 
