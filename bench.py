@@ -10,7 +10,9 @@ roofline fraction of each point), beside the peaks two measuring kernels of the 
 this GPU.  ``--profile`` adds, on stderr, milliseconds / bytes / GB/s per kernel class of one
 prefill and one decode step, from event pairs.  ``--shape maverick8`` and ``--shape long16`` run
 two other workloads instead (128 experts alternating with dense layers at batch 64; 32,768-token
-prompts read in 4,096-token portions beside decoding requests) and print a JSON line of their own.
+prompts read in 4,096-token portions beside decoding requests) and print a JSON line of their own;
+``--shape kuvonex`` runs Kuvonex layers (latent attention, routed experts in groups) at two sizes,
+each beside Llama 4 layers of the same width, heads and experts, with the kernel-class tables of both.
 """
 from __future__ import annotations
 

@@ -117,10 +117,10 @@ def latent_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], p: str, mx: di
 
 
 def route(h: torch.Tensor, w_router: torch.Tensor, correction: torch.Tensor, router: dict, ids=None):
-    """Picks and weights (`ids` given: only the weights of those picks are made).  s = sigmoid(W_router h); experts are chosen by s + correction, among
-    the experts of the `keep` best groups only (a group's rank: the sum of its GROUP_TOP largest
+    """Picks and weights.  s = sigmoid(W_router h); experts are chosen by s + correction, among the
+    experts of the `keep` best groups only (a group's rank: the sum of its GROUP_TOP largest
     choice scores); the weights are s of the chosen, as they are.  Returns ids [T, top] (best
-    first), weights [T, top]."""
+    first), weights [T, top].  With `ids` given, only the weights of those picks are made."""
     E, top = int(router["experts"]), int(router["top"])
     s = torch.sigmoid(h @ w_router.T)
     if ids is not None:
