@@ -171,3 +171,20 @@ def test_a_prefix_gives_the_logits_of_the_whole():
     whole, layers = P.forward(c, w, toks, want_layers=True)
     part = P.forward(c, w, toks[:6])
     assert torch.allclose(whole[:6], part, atol=1e-9) and layers.shape == (4, len(toks), 64)
+
+
+def test_the_benchmark_shapes_are_valid_configurations_of_both_architectures():
+    import importlib.util
+    import os
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("bench_for_test", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    for z in bench.KUVONEX_SIZES.values():
+        k = load_config(bench.kuvonex_config(z))
+        l = load_config(bench.llama4_config_like(z))
+        assert k.width == l.hidden_size == z["width"] and len(k.layers) == l.num_hidden_layers == z["layers"]
+        assert k.layers[0].mlp.experts == l.num_local_experts and k.layers[0].mlp.ff == l.intermediate_size
+        assert k.layers[-1].mixer.kv_from == z["layers"] - 2 and k.layers[0].mixer.kv_from is None
+        build_model(k), build_model(l)
