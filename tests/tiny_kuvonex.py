@@ -43,8 +43,22 @@ EVEN = {
     ],
 }
 
-CONFIGS = {"odd": ODD, "even": EVEN}
-SEEDS = {"odd": 11, "even": 12}
+# five layers of five shapes: a latent of 80 beside rows of 104 (the matrix cores take them), two caches shared
+# in different ways, twelve heads over a latent of 48, one head with a rotated part of two elements, groups of
+# one expert, every group kept, a width that is no multiple of 64
+MID = {
+    "architecture": "Kuvonex", "vocab": 211, "width": 96, "norm": {"eps": 1e-5}, "embedding": {"scale": 7.0},
+    "layers": [
+        _layer(_mixer(6, 40, 24, 56, 80, 0.11, 10000.0), _moe(12, 4, 80, (3, 2))),
+        _layer(_mixer(2, 64, 24, 8, 80, 0.2, 10000.0, kv_from=0), _moe(5, 2, 30)),
+        _layer(_mixer(4, 16, 8, 16, 48, 0.3, 300.0), None),
+        _layer(_mixer(12, 32, 8, 32, 48, 0.1, 300.0, kv_from=2), _moe(9, 3, 64, (9, 9))),
+        _layer(_mixer(1, 128, 2, 64, 16, 0.05, 1.0e6), _moe(2, 1, 48, (2, 1))),
+    ],
+}
+
+CONFIGS = {"odd": ODD, "even": EVEN, "mid": MID}
+SEEDS = {"odd": 11, "even": 12, "mid": 13}
 # sinks and corrections large enough that leaving one out shows
 STD_BY_SUFFIX = {".sink": 1.5, ".correction": 0.4}
 
