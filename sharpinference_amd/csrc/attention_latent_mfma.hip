@@ -377,6 +377,7 @@ SHARPI_EXPORT int sharpi_attention_latent_mfma(const void* q, const void* rows, 
   } while (0)
   if (g.d32 <= 5 && g.r16 <= 8) LM_LAUNCH(5, 8);
   else if (g.d32 <= 10 && g.r16 <= 16) LM_LAUNCH(10, 16);
+  else if (g.d32 <= 18) LM_LAUNCH(18, 32);      // rows of up to 576: eight registers fewer than the widest form, which spills
   else LM_LAUNCH(20, 32);
 #undef LM_LAUNCH
   SHARPI_CHECK_LAUNCH();
