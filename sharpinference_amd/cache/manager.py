@@ -22,7 +22,7 @@ from typing import Dict, Hashable, List, Optional, Sequence, Union
 import numpy as np
 import torch
 
-from .spec import KVSpec, StateSpec
+from .spec import KVSpec, MixedSpec, StateSpec, kv_of, states_of
 
 
 class CacheError(RuntimeError):
@@ -48,7 +48,8 @@ def pool_sizes(slot_specs, page_size: int, max_requests: int, total_tokens: int,
     can ever hold, which is what makes its memory bounded however long the requests grow."""
     out: Dict[tuple, int] = {}
     for spec in slot_specs:
-        if not isinstance(spec, KVSpec) or spec.group_key() in out:
+        spec = kv_of(spec)
+        if spec is None or spec.group_key() in out:
             continue
         n = max_requests * pages_to_hold(spec, page_size, total_tokens, max_step_tokens)
         if budget_pages is not None:
@@ -112,7 +113,7 @@ class RequestCache:
 
 
 class CacheManager:
-    def __init__(self, slot_specs: Sequence[Union[KVSpec, StateSpec, None]], page_size: int,
+    def __init__(self, slot_specs: Sequence[Union[KVSpec, StateSpec, MixedSpec, None]], page_size: int,
                  num_pages: Union[int, Dict[tuple, int]], max_requests: int, dtype: torch.dtype = torch.float32,
                  device="cpu", allocate: bool = True):
         if page_size <= 0 or page_size % 16 != 0:
@@ -128,7 +129,8 @@ class CacheManager:
         self.group_of_slot: List[int] = []
         by_key: Dict[tuple, int] = {}
         for i, spec in enumerate(self.slot_specs):
-            if isinstance(spec, KVSpec):
+            spec = kv_of(spec)
+            if spec is not None:
                 key = spec.group_key()
                 if key not in by_key:
                     n = num_pages[key] if isinstance(num_pages, dict) else int(num_pages)
@@ -148,10 +150,14 @@ class CacheManager:
         # device tensors
         self.k: List[Optional[torch.Tensor]] = [None] * len(self.slot_specs)
         self.v: List[Optional[torch.Tensor]] = [None] * len(self.slot_specs)
+        # fixed-size states: per cache slot, one tensor per StateSpec the layer asked for, in its order
+        # (`state` is the first of them, what a mixer with a single state reads)
+        self.states: List[List[torch.Tensor]] = [[] for _ in self.slot_specs]
         self.state: List[Optional[torch.Tensor]] = [None] * len(self.slot_specs)
         if allocate:
-            for i, spec in enumerate(self.slot_specs):
-                if isinstance(spec, KVSpec):
+            for i, whole in enumerate(self.slot_specs):
+                spec = kv_of(whole)
+                if spec is not None:
                     n = self.groups[self.group_of_slot[i]].pool.num_pages
                     # keys [page, kv head, position, head_dim]; values transposed inside the page,
                     # [page, kv head, head_dim, position], the layout the matrix-core kernels read
@@ -160,8 +166,10 @@ class CacheManager:
                     if not spec.values_in_keys:
                         self.v[i] = torch.zeros((n, spec.num_kv_heads, spec.value_dim, page_size), dtype=dtype,
                                                 device=self.device)
-                elif isinstance(spec, StateSpec):
-                    self.state[i] = torch.zeros((max_requests + 1, *spec.shape), dtype=spec.dtype, device=self.device)
+                for st in states_of(whole):
+                    self.states[i].append(torch.zeros((max_requests + 1, *st.shape), dtype=st.dtype, device=self.device))
+                if self.states[i]:
+                    self.state[i] = self.states[i][0]
 
     # ------------------------------------------------------------------ sizes
     def bytes_per_page(self) -> List[int]:
@@ -171,7 +179,7 @@ class CacheManager:
         for g in self.groups:
             b = 0
             for s in g.slots:
-                spec = self.slot_specs[s]
+                spec = kv_of(self.slot_specs[s])
                 b += spec.elements_per_token * self.page_size * width
             out.append(b)
         return out
@@ -221,8 +229,8 @@ class CacheManager:
                 rc.reserved[g] = self.pages_to_hold(g, reserve_tokens, max_step_tokens)
                 self._reserved_total[g] += rc.reserved[g]
         rc.state_slot = self._free_state_slots.pop()
-        for t in self.state:
-            if t is not None:
+        for per_slot in self.states:
+            for t in per_slot:
                 t[rc.state_slot].zero_()
         self.requests[req_id] = rc
         return rc

@@ -5,12 +5,15 @@ sequence, kept in pages; a window tells which of them a later query can still se
 pages behind it go back to the pool.  ``StateSpec``: a block of fixed size per request (a
 recurrent state, a convolution tail), kept in a slot
 (reference: src/SharpInference.Engine/GdnStateCache.cs:7-33 for the fixed-size kind,
-src/SharpInference.Engine/PagedKvCache.cs:20-110 for the paged kind).
+src/SharpInference.Engine/PagedKvCache.cs:20-110 for the paged kind).  A mixer that needs both
+(attention behind short convolutions; attention beside a recurrent mixer) asks with a
+``MixedSpec``: at most one ``KVSpec`` and any number of ``StateSpec``, which it finds again in
+the order it gave them.
 """
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Tuple
+from typing import Optional, Tuple
 
 import torch
 
@@ -59,3 +62,44 @@ class StateSpec:
 
     def group_key(self):
         return ("state",)
+
+
+@dataclass(frozen=True)
+class MixedSpec:
+    """Paged keys and values and fixed-size states of one layer together."""
+
+    kv: Optional[KVSpec]
+    states: Tuple[StateSpec, ...] = ()
+
+    def group_key(self):
+        return self.kv.group_key() if self.kv is not None else ("state",)
+
+
+def kv_of(spec) -> Optional[KVSpec]:
+    """The paged part of what a layer asks for, if it has one."""
+    if isinstance(spec, KVSpec):
+        return spec
+    return spec.kv if isinstance(spec, MixedSpec) else None
+
+
+def states_of(spec) -> Tuple[StateSpec, ...]:
+    """The fixed-size states a layer asks for, in its order."""
+    if isinstance(spec, StateSpec):
+        return (spec,)
+    return tuple(spec.states) if isinstance(spec, MixedSpec) else ()
+
+
+def combine_specs(specs) -> object:
+    """One request for the memory of several mixers that share a layer: the one paged part among
+    them and all their states, in order.  None if none of them keeps anything."""
+    kvs = [kv_of(s) for s in specs if kv_of(s) is not None]
+    if len(kvs) > 1:
+        raise ValueError("a layer can hold the pages of one mixer only")
+    states = tuple(st for s in specs for st in states_of(s))
+    if not kvs and not states:
+        return None
+    if not states:
+        return kvs[0]
+    if not kvs and len(states) == 1:
+        return states[0]
+    return MixedSpec(kvs[0] if kvs else None, states)

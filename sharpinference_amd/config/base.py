@@ -50,6 +50,11 @@ class ModelConfig:
     def validate(self) -> None:
         """Raise ConfigError when sizes or options contradict each other."""
 
+    def with_tensor_shapes(self, available: Dict[str, tuple]) -> "ModelConfig":
+        """The configuration completed by sizes that no key of config.json gives and a tensor's
+        shape does (`available`: name -> (shape, dtype) of a weight file).  Most designs have none."""
+        return self
+
     def special_tokens_dict(self) -> Dict[str, Any]:
         """The token keys as config.json writes them (absent where the configuration has none)."""
         out: Dict[str, Any] = {}

@@ -41,7 +41,7 @@ __global__ __launch_bounds__(kDecWaves* kWave) void attn_decode_kernel(
     const int* __restrict__ block_table, const int* __restrict__ entry_of_token,
     const int* __restrict__ positions, const int* __restrict__ token_list, float* __restrict__ part_o,
     float* __restrict__ part_ml, int window_kind, int window, float scale, int nh, int nkv, int page_size,
-    int max_blocks, int num_pages, int max_splits) {
+    int max_blocks, int num_pages, int max_splits, float softcap) {
   constexpr int NJ = HD / 32;  // 32-wide d chunks of the first product
   constexpr int ND = HD / 16;  // 16-row d tiles of the second product
   __shared__ f32x4 acc_s[kDecWaves][ND][kWave];
@@ -136,7 +136,9 @@ __global__ __launch_bounds__(kDecWaves* kWave) void attn_decode_kernel(
       for (int i = 0; i < 4; ++i) {
         const int key = ((b + u) << 4) + 4 * g + i;
         const bool ok = have[u] && key >= start && key <= p;
-        s[u][i] = ok ? s[u][i] * scale : -INFINITY;
+        float sc = s[u][i] * scale;
+        if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);   // (uniform: a layer either caps its scores or not)
+        s[u][i] = ok ? sc : -INFINITY;
         cm = fmaxf(cm, s[u][i]);
       }
     cm = fmaxf(cm, __shfl_xor(cm, 16, kWave));
@@ -216,7 +218,7 @@ constexpr int kMergeThreads = 256;
 __global__ __launch_bounds__(kMergeThreads) void attn_decode_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ positions,
     const int* __restrict__ token_list, bf16_t* __restrict__ out, int window_kind, int window, int nh, int hd,
-    int max_splits) {
+    int max_splits, int sink) {
   __shared__ float red_s[kMergeThreads / kWave];
   __shared__ f32x4 o_s[kMergeThreads];
   __shared__ float l_s[kMergeThreads];
@@ -267,6 +269,7 @@ __global__ __launch_bounds__(kMergeThreads) void attn_decode_merge_kernel(
     o += o_s[x * ncol + col];
     L += l_s[x * ncol + col];
   }
+  if (sink && M > -INFINITY) L += expf(-M);   // a key of score 0 without a value: one more term in the denominator
   unsigned short b[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) b[i] = runs_wanted > max_splits ? (unsigned short)0x7fc0 : f32_to_bf16(L > 0.f ? o[i] / L : 0.f).bits;
@@ -280,17 +283,18 @@ template <int HD>
 static int launch_decode(const void* q, const void* k_cache, const void* v_cache, const int* block_table,
                          const int* entry_of_token, const int* positions, const int* token_list, float* part_o,
                          float* part_ml, void* out, int window_kind, int window, float scale, int n_list, int nh,
-                         int nkv, int page_size, int max_blocks, int num_pages, int max_splits, hipStream_t stream) {
+                         int nkv, int page_size, int max_blocks, int num_pages, int max_splits, float softcap, int sink,
+                         hipStream_t stream) {
   const int G = nh / nkv;
   dim3 grid(nkv * ((G + 15) / 16), n_list, max_splits), block(kDecWaves * kWave);
   attn_decode_kernel<HD><<<grid, block, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
                                                     block_table, entry_of_token, positions, token_list, part_o,
                                                     part_ml, window_kind, window, scale, nh, nkv, page_size,
-                                                    max_blocks, num_pages, max_splits);
+                                                    max_blocks, num_pages, max_splits, softcap);
   SHARPI_CHECK_LAUNCH();
   dim3 mgrid(n_list, nh), mblock(kMergeThreads);
   attn_decode_merge_kernel<<<mgrid, mblock, 0, stream>>>(part_o, part_ml, positions, token_list, (bf16_t*)out,
-                                                         window_kind, window, nh, HD, max_splits);
+                                                         window_kind, window, nh, HD, max_splits, sink);
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }
@@ -301,23 +305,24 @@ static int launch_decode(const void* q, const void* k_cache, const void* v_cache
 // max_splits must cover every listed token: ((position >> 4) - (first visible key >> 4)) / 16 + 1
 // runs of 256 keys (runs are aligned to absolute positions, so a window that starts inside a run
 // takes one more than its length suggests); ((context - 1) >> 4) / 16 + 1 covers every window of a
-// context.  A token whose runs exceed max_splits gets a row of NaN.
+// context.  A token whose runs exceed max_splits gets a row of NaN.  softcap > 0: scores become
+// softcap * tanh(score / softcap); sink: the denominator holds one more term exp(0).
 SHARPI_EXPORT int sharpi_attention_decode(const void* q, const void* k_cache, const void* v_cache,
                                           const int* block_table, const int* entry_of_token, const int* positions,
                                           const int* token_list, float* part_o, float* part_ml, void* out,
                                           int window_kind, int window, float scale, int n_list, int nh, int nkv,
                                           int hd, int page_size, int max_blocks, int num_pages, int max_splits,
-                                          hipStream_t stream) {
+                                          float softcap, int sink, hipStream_t stream) {
   if (n_list <= 0) return SHARPI_OK;
   if (nh <= 0 || nkv <= 0 || nh % nkv != 0 || nh > 65535 || n_list > 65535) return SHARPI_ERR_ARG;
   if (page_size <= 0 || page_size % 16 != 0 || max_blocks <= 0 || num_pages <= 0 || max_splits <= 0 || max_splits > 65535) return SHARPI_ERR_ARG;
-  if (window_kind < 0 || window_kind > 2 || (window_kind != 0 && window <= 0)) return SHARPI_ERR_ARG;
+  if (window_kind < 0 || window_kind > 2 || (window_kind != 0 && window <= 0) || !(softcap >= 0.f)) return SHARPI_ERR_ARG;
   if (nkv * ((nh / nkv + 15) / 16) > 65535) return SHARPI_ERR_ARG;
 #define DEC(HDV)                                                                                                  \
   if (hd == HDV)                                                                                                  \
     return launch_decode<HDV>(q, k_cache, v_cache, block_table, entry_of_token, positions, token_list, part_o,    \
                               part_ml, out, window_kind, window, scale, n_list, nh, nkv, page_size, max_blocks,   \
-                              num_pages, max_splits, stream);
+                              num_pages, max_splits, softcap, sink, stream);
   SHARPI_DECODE_HEAD_SIZES(DEC)
 #undef DEC
   return SHARPI_ERR_ARG;  // other head sizes go to the generic kernel
@@ -377,5 +382,5 @@ int sharpi_attention_decode_noalloc(const void* q, const void* k_cache, const vo
   float* part_ml = ws + runs * (unsigned long long)hd;   // hd is a multiple of 32: stays 16-byte aligned
   return sharpi_attention_decode(q, k_cache, v_cache, block_table, entry_of_token, positions, token_list, part_o,
                                  part_ml, out, window_kind, window, scale, n_list, nh, nkv, hd, page_size, max_blocks,
-                                 num_pages, max_splits, stream);
+                                 num_pages, max_splits, 0.f, 0, stream);
 }

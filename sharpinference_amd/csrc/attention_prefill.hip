@@ -74,7 +74,7 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? (kQT == 1 ? 3 : 2) : 
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_table, const int* __restrict__ positions, const int* __restrict__ tiles,
     bf16_t* __restrict__ out, int window_kind, int window, float scale, int nh, int nkv, int page_size,
-    int max_blocks, int num_pages) {
+    int max_blocks, int num_pages, float softcap, int sink) {
   constexpr int kWaveTokens = 16 * kQT;
   constexpr int NJ = HD / 32;
   constexpr int ND = HD / 16;
@@ -128,6 +128,8 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? (kQT == 1 ? 3 : 2) : 
   if (window_kind == 1) wave_last_start = (wave_last / window) * window;
   else if (window_kind == 2) wave_last_start = wave_last - window + 1 > 0 ? wave_last - window + 1 : 0;
   const float scale_log2 = scale * 1.4426950408889634f;               // softmax in base 2: exp(x) = 2^(x log2 e)
+  const float cap_log2 = softcap * 1.4426950408889634f;               // capped scores: cap * tanh(score / cap), in base-2 units
+  const float scale_by_cap = softcap > 0.f ? scale / softcap : 0.f;
   int wave_first = pos0 + wrow0;                                      // first key the wave's first row may see
   if (window_kind == 1) wave_first = (wave_first / window) * window;
   else if (window_kind == 2) wave_first = wave_first - window + 1 > 0 ? wave_first - window + 1 : 0;
@@ -279,7 +281,7 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? (kQT == 1 ? 3 : 2) : 
         for (int u = 0; u < 2; ++u)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            float t = s[c][u][i] * scale_log2;
+            float t = softcap > 0.f ? cap_log2 * tanhf(s[c][u][i] * scale_by_cap) : s[c][u][i] * scale_log2;
             if (!whole) {
               const int key = ((b + u) << 4) + 4 * g + i;
               const bool ok = have[u] && qok[c] && key >= qstart[c] && key <= qpos[c];
@@ -369,6 +371,7 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? (kQT == 1 ? 3 : 2) : 
     L += __shfl_xor(L, 16, kWave);
     L += __shfl_xor(L, 32, kWave);
     if (!qok[c]) continue;
+    if (sink) L += __builtin_amdgcn_exp2f(-m[c]);   // a key of score 0 without a value: 2^(0 - reference) more
     const float inv = L > 0.f ? 1.0f / L : 0.f;
     bf16_t* orow = out + ((size_t)(tok0 + wrow0 + c * 16 + r) * nh + h) * HD;
 #pragma unroll
@@ -386,23 +389,24 @@ __global__ __launch_bounds__(kPreWaves* kWave, HD <= 128 ? (kQT == 1 ? 3 : 2) : 
 // q [T, nh, hd] bf16; caches K [pages, nkv, page_size, hd], V [pages, nkv, hd, page_size] bf16;
 // tiles int32 [n_tiles, 3] = (entry, first token, rows <= tile_tokens), tokens of a tile consecutive
 // in one entry; tile_tokens 128 or 64 (what the caller cut the tiles to: no tile may hold more);
-// out [T, nh, hd] bf16 (rows of the listed tiles).
+// out [T, nh, hd] bf16 (rows of the listed tiles).  softcap > 0: scores become softcap * tanh(score /
+// softcap); sink: the denominator holds one more term exp(0).
 SHARPI_EXPORT int sharpi_attention_prefill(const void* q, const void* k_cache, const void* v_cache,
                                            const int* block_table, const int* positions, const int* tiles,
                                            void* out, int n_tiles, int tile_tokens, int window_kind, int window,
                                            float scale, int nh, int nkv, int hd, int page_size, int max_blocks,
-                                           int num_pages, hipStream_t stream) {
+                                           int num_pages, float softcap, int sink, hipStream_t stream) {
   if (n_tiles <= 0) return SHARPI_OK;
   if (nh <= 0 || nkv <= 0 || nh % nkv != 0 || n_tiles > 65535) return SHARPI_ERR_ARG;
   if (tile_tokens != kTileTokens && tile_tokens != kTileTokens / 2) return SHARPI_ERR_ARG;
   if (page_size <= 0 || page_size % 16 != 0 || max_blocks <= 0 || num_pages <= 0) return SHARPI_ERR_ARG;
-  if (window_kind < 0 || window_kind > 2 || (window_kind != 0 && window <= 0)) return SHARPI_ERR_ARG;
+  if (window_kind < 0 || window_kind > 2 || (window_kind != 0 && window <= 0) || !(softcap >= 0.f)) return SHARPI_ERR_ARG;
   dim3 grid(nh, n_tiles), block(kPreWaves * kWave);
 #define PRE_QT(HDV, QTV)                                                                                        \
   attn_prefill_kernel<HDV, QTV><<<grid, block, 0, stream>>>((const bf16_t*)q, (const bf16_t*)k_cache,               \
                                                            (const bf16_t*)v_cache, block_table, positions, tiles,  \
                                                            (bf16_t*)out, window_kind, window, scale, nh, nkv,      \
-                                                           page_size, max_blocks, num_pages)
+                                                           page_size, max_blocks, num_pages, softcap, sink)
 #define PRE(HDV)                                  \
   if (hd == HDV) {                                \
     if (tile_tokens == kTileTokens) PRE_QT(HDV, 2); \

@@ -451,3 +451,86 @@ SHARPI_EXPORT int sharpi_scale_softcap(float* x, long long n, float scale, float
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }
+
+// ---------------------------------------------------------------------------
+// An ungated activation, element by element: out = f(x).  f: 1 the square of relu; 2 tanh-GELU;
+// 3 SiLU.  For feed-forwards without a gate (down(f(up x))).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void activation_kernel(const T* __restrict__ x, T* __restrict__ out, size_t n, int f) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const float v = to_f32<T>(x[i]);
+    float y;
+    if (f == 1) {
+      const float r = fmaxf(v, 0.f);
+      y = r * r;
+    } else if (f == 2) {
+      y = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+    } else {
+      y = v / (1.0f + expf(-v));
+    }
+    out[i] = from_f32<T>(y);
+  }
+}
+
+SHARPI_EXPORT int sharpi_activation(const void* x, void* out, int dtype, long long n, int f, hipStream_t stream) {
+  if (n <= 0) return SHARPI_OK;
+  if (f < 1 || f > 3) return SHARPI_ERR_ARG;
+  const dim3 block(256), grid((unsigned)min((long long)8192, (n + 255) / 256));
+  if (dtype == DT_F32) activation_kernel<float><<<grid, block, 0, stream>>>((const float*)x, (float*)out, (size_t)n, f);
+  else if (dtype == DT_BF16) activation_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, (size_t)n, f);
+  else return SHARPI_ERR_ARG;
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Branches that run side by side on the same input, joined: out[t] = (1 / n) * sum_b
+// unit_rms(x_b[t]) * w_b, each branch normed over the row with its own learned weights.  One block
+// a row; statistics and the sum in float; out float [T, N].  Up to four branches.
+// ---------------------------------------------------------------------------
+constexpr int kMaxBranches = 4;
+struct BranchArgs {
+  const void* x[kMaxBranches];
+  const float* w[kMaxBranches];
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void norm_mean_kernel(BranchArgs a, int n_branches, float* __restrict__ out, int N,
+                                                        float eps) {
+  __shared__ float red[16];
+  const size_t t = blockIdx.x;
+  float inv[kMaxBranches];
+  for (int b = 0; b < n_branches; ++b) {
+    const T* x = (const T*)a.x[b] + t * N;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < N; i += blockDim.x) {
+      const float v = to_f32<T>(x[i]);
+      ss = fmaf(v, v, ss);
+    }
+    inv[b] = rsqrtf(block_sum(ss, red) / (float)N + eps);
+  }
+  const float share = 1.0f / (float)n_branches;
+  for (int i = threadIdx.x; i < N; i += blockDim.x) {
+    float y = 0.f;
+    for (int b = 0; b < n_branches; ++b) y += to_f32<T>(((const T*)a.x[b])[t * N + i]) * inv[b] * a.w[b][i];
+    out[t * N + i] = y * share;
+  }
+}
+
+SHARPI_EXPORT int sharpi_norm_mean(const void* const* xs, const float* const* ws, int n_branches, int dtype, void* out,
+                                   int n_rows, int N, float eps, hipStream_t stream) {
+  if (n_rows <= 0) return SHARPI_OK;
+  if (n_branches < 1 || n_branches > kMaxBranches || N <= 0) return SHARPI_ERR_ARG;
+  BranchArgs a{};
+  for (int b = 0; b < n_branches; ++b) {
+    if (!xs[b] || !ws[b]) return SHARPI_ERR_ARG;
+    a.x[b] = xs[b];
+    a.w[b] = ws[b];
+  }
+  if (dtype == DT_F32) norm_mean_kernel<float><<<n_rows, 256, 0, stream>>>(a, n_branches, (float*)out, N, eps);
+  else if (dtype == DT_BF16) norm_mean_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(a, n_branches, (float*)out, N, eps);
+  else return SHARPI_ERR_ARG;
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}

@@ -1,0 +1,225 @@
+// What lies between an attention layer's input projections and its attention kernel, for layers
+// that norm before they rotate: an optional short causal convolution over time on every channel
+// of q, k and v, an RMS norm of q and of k with learned weights (per head, one weight vector
+// shared by the heads; or over the whole projection, one weight per channel), rotary positions on
+// the first r elements of every head (pairs interleaved or split in halves, cos and sin times a
+// magnitude), and the write of keys and values into the paged cache.  Values may be the keys as
+// they were before norm and rotation (a layer without a value projection).
+//
+// One block per token.  The token's row is gathered into LDS as floats (the convolution reads up
+// to taps - 1 earlier rows: of this step where the entry has them, otherwise the tail that the
+// request's state slot carries), the sums of squares are taken in an order that depends on the
+// row alone, and everything after the projection is float arithmetic rounded once, on the way out.
+#include "common.h"
+
+constexpr int kPrepThreads = 256;
+constexpr int kPrepMaxTaps = 8;
+constexpr int kPrepMaxHeads = 1024;   // q heads + kv heads whose inverse norms are kept in LDS
+
+enum : int { NORM_NONE = 0, NORM_PER_HEAD = 1, NORM_WHOLE = 2 };
+
+struct PrepArgs {
+  const void* proj;        // [T, stride]
+  int stride, q_off, k_off, v_off;   // v_off < 0: the values are the keys before norm and rotation
+  int nh, nkv, hd, vd;
+  const float* conv_w;     // [q + k + v channels, taps] or null
+  int taps;
+  float* tail;             // [slots, taps - 1, channels]: the last projected rows of each request
+  const int* state_slots;  // [entries]
+  const int* entry_of_token;
+  const int* cu_tokens;
+  const int* positions;
+  int norm_mode;
+  const float* q_norm_w;   // [hd] or [nh * hd]
+  const float* k_norm_w;   // [hd] or [nkv * hd]
+  float eps;
+  const float* inv_freq;   // [rotary_dim / 2] or null
+  int rotary_dim, half_split;
+  float magnitude;
+  void* q_out;             // [T, nh * hd]
+  void* k_cache;           // [pages, nkv, page_size, hd]
+  void* v_cache;           // [pages, nkv, vd, page_size]
+  const int* slot_mapping; // [T], -1: store nothing
+  int page_size;
+};
+
+template <typename T>
+__global__ __launch_bounds__(kPrepThreads) void qk_prep_kernel(PrepArgs a) {
+  extern __shared__ float row[];          // q | k | v of the token, as floats
+  __shared__ float red[16];
+  __shared__ float inv[kPrepMaxHeads];
+  const int t = blockIdx.x;
+  const int qn = a.nh * a.hd, kn = a.nkv * a.hd;
+  const bool own_v = a.v_off >= 0;
+  const int vn = own_v ? a.nkv * a.vd : 0;
+  const int C = qn + kn + vn;
+  const T* proj = (const T*)a.proj;
+
+  // 1. gather, through the convolution where there is one
+  if (a.taps > 0) {
+    const int e = a.entry_of_token[t];
+    const int li = t - a.cu_tokens[e];                 // the token's place in its entry
+    const float* tail = a.tail + (size_t)a.state_slots[e] * (a.taps - 1) * C;
+    for (int c = threadIdx.x; c < C; c += kPrepThreads) {
+      const int col = c < qn ? a.q_off + c : c < qn + kn ? a.k_off + (c - qn) : a.v_off + (c - qn - kn);
+      float y = 0.f;
+      for (int j = 0; j < a.taps; ++j) {
+        const int back = a.taps - 1 - j;               // this tap reads the row `back` tokens ago
+        float u;
+        if (back <= li) u = to_f32<T>(proj[(size_t)(t - back) * a.stride + col]);
+        else u = tail[(size_t)(a.taps - 1 + li - back) * C + c];
+        y = fmaf(a.conv_w[(size_t)c * a.taps + j], u, y);
+      }
+      row[c] = y;
+    }
+  } else {
+    for (int c = threadIdx.x; c < C; c += kPrepThreads) {
+      const int col = c < qn ? a.q_off + c : c < qn + kn ? a.k_off + (c - qn) : a.v_off + (c - qn - kn);
+      row[c] = to_f32<T>(proj[(size_t)t * a.stride + col]);
+    }
+  }
+  __syncthreads();
+
+  // 2. values leave as they are (a layer without a value projection stores its unnormed keys)
+  const int slot = a.slot_mapping ? a.slot_mapping[t] : -1;
+  if (slot >= 0) {
+    const int page = slot / a.page_size, off = slot % a.page_size;
+    T* vc = (T*)a.v_cache;
+    const float* vsrc = own_v ? row + qn + kn : row + qn;
+    for (int i = threadIdx.x; i < a.nkv * a.vd; i += kPrepThreads) {
+      const int g = i / a.vd, d = i % a.vd;
+      vc[(((size_t)page * a.nkv + g) * a.vd + d) * a.page_size + off] = from_f32<T>(vsrc[i]);
+    }
+  }
+
+  // 3. inverse norms
+  const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x >> 6;
+  const int heads = a.nh + a.nkv;
+  if (a.norm_mode == NORM_PER_HEAD) {
+    for (int h = wid; h < heads; h += kPrepThreads / kWave) {
+      const float* x = row + (size_t)h * a.hd;         // (q heads then k heads lie back to back)
+      float ss = 0.f;
+      for (int d = lane; d < a.hd; d += kWave) ss = fmaf(x[d], x[d], ss);
+      ss = wave_sum(ss);
+      if (lane == 0) inv[h] = rsqrtf(ss / (float)a.hd + a.eps);
+    }
+  } else if (a.norm_mode == NORM_WHOLE) {
+    float sq = 0.f, sk = 0.f;
+    for (int c = threadIdx.x; c < qn; c += kPrepThreads) sq = fmaf(row[c], row[c], sq);
+    for (int c = threadIdx.x; c < kn; c += kPrepThreads) sk = fmaf(row[qn + c], row[qn + c], sk);
+    sq = block_sum(sq, red);
+    sk = block_sum(sk, red);
+    const float iq = rsqrtf(sq / (float)qn + a.eps), ik = rsqrtf(sk / (float)kn + a.eps);
+    for (int h = threadIdx.x; h < heads; h += kPrepThreads) inv[h] = h < a.nh ? iq : ik;
+  }
+  __syncthreads();
+
+  // 4. norm, rotation, and out: a thread takes a pair of a head (or two elements that do not turn)
+  const float pos = (float)a.positions[t];
+  const int half_hd = a.hd / 2, half_r = a.rotary_dim / 2;
+  T* qo = (T*)a.q_out + (size_t)t * qn;
+  T* kc = (T*)a.k_cache;
+  for (int i = threadIdx.x; i < heads * half_hd; i += kPrepThreads) {
+    const int h = i / half_hd, pi = i % half_hd;
+    int d0, d1;
+    bool turns;
+    if (pi < half_r) {
+      turns = true;
+      d0 = a.half_split ? pi : 2 * pi;
+      d1 = a.half_split ? pi + half_r : 2 * pi + 1;
+    } else {
+      turns = false;
+      d0 = a.rotary_dim + 2 * (pi - half_r);
+      d1 = d0 + 1;
+    }
+    const bool is_q = h < a.nh;
+    float x0 = row[(size_t)h * a.hd + d0], x1 = row[(size_t)h * a.hd + d1];
+    if (a.norm_mode != NORM_NONE) {
+      const float* w = is_q ? a.q_norm_w : a.k_norm_w;
+      const int wbase = a.norm_mode == NORM_WHOLE ? (is_q ? h : h - a.nh) * a.hd : 0;
+      x0 = x0 * inv[h] * w[wbase + d0];
+      x1 = x1 * inv[h] * w[wbase + d1];
+    }
+    if (turns && a.inv_freq) {
+      const float ang = pos * a.inv_freq[pi];
+      const float c = cosf(ang) * a.magnitude, s = sinf(ang) * a.magnitude;
+      const float y0 = x0 * c - x1 * s, y1 = x1 * c + x0 * s;
+      x0 = y0;
+      x1 = y1;
+    }
+    if (is_q) {
+      qo[(size_t)h * a.hd + d0] = from_f32<T>(x0);
+      qo[(size_t)h * a.hd + d1] = from_f32<T>(x1);
+    } else if (slot >= 0) {
+      const int page = slot / a.page_size, off = slot % a.page_size;
+      T* kr = kc + (((size_t)page * a.nkv + (h - a.nh)) * a.page_size + off) * a.hd;
+      kr[d0] = from_f32<T>(x0);
+      kr[d1] = from_f32<T>(x1);
+    }
+  }
+}
+
+// The convolution's tail after a step: the last taps - 1 projected rows of each entry's request
+// (rows of this step where the entry brought enough, what the slot held before otherwise).  A
+// thread takes one channel of one entry, reads everything it needs and only then writes.
+template <typename T>
+__global__ void conv_tail_kernel(const T* __restrict__ proj, int stride, int q_off, int k_off, int v_off, int qn, int kn,
+                                 int vn, int taps, float* __restrict__ tail, const int* __restrict__ state_slots,
+                                 const int* __restrict__ cu_tokens) {
+  const int e = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int C = qn + kn + vn;
+  if (c >= C) return;
+  const int col = c < qn ? q_off + c : c < qn + kn ? k_off + (c - qn) : v_off + (c - qn - kn);
+  const int first = cu_tokens[e], len = cu_tokens[e + 1] - first;
+  float* mine = tail + (size_t)state_slots[e] * (taps - 1) * C + c;
+  float keep[kPrepMaxTaps];
+  for (int s = 0; s < taps - 1; ++s) {
+    const int li = len - (taps - 1) + s;               // the row that ends up in place s
+    keep[s] = li >= 0 ? to_f32<T>(proj[(size_t)(first + li) * stride + col]) : mine[(size_t)(taps - 1 + li) * C];
+  }
+  for (int s = 0; s < taps - 1; ++s) mine[(size_t)s * C] = keep[s];
+}
+
+// proj [T, stride] of `dtype`; q at columns q_off.., k at k_off.., v at v_off.. (v_off < 0: values
+// are the unnormed keys, vd must equal hd).  conv_w float [channels, taps] (taps 0: none), tail float
+// [slots, taps - 1, channels].  norm_mode 0 none / 1 per head (weights [hd]) / 2 whole projection
+// (weights [nh*hd], [nkv*hd]).  inv_freq float [rotary_dim / 2] or null.  Caches K [pages, nkv,
+// page_size, hd], V [pages, nkv, vd, page_size]; slot_mapping null or -1: nothing is stored.
+SHARPI_EXPORT int sharpi_qk_prep(const void* proj, int dtype, int stride, int q_off, int k_off, int v_off, int n_tokens,
+                                 int n_entries, int nh, int nkv, int hd, int vd, const float* conv_w, int taps, float* tail,
+                                 const int* state_slots, const int* entry_of_token, const int* cu_tokens,
+                                 const int* positions, int norm_mode, const float* q_norm_w, const float* k_norm_w,
+                                 float eps, const float* inv_freq, int rotary_dim, int half_split, float magnitude,
+                                 void* q_out, void* k_cache, void* v_cache, const int* slot_mapping, int page_size,
+                                 int update_tail, hipStream_t stream) {
+  if (n_tokens <= 0) return SHARPI_OK;
+  if (nh <= 0 || nkv <= 0 || hd <= 0 || hd % 2 || vd <= 0 || nh + nkv > kPrepMaxHeads) return SHARPI_ERR_ARG;
+  if (taps < 0 || taps == 1 || taps > kPrepMaxTaps || (taps > 0 && (!conv_w || !tail || !state_slots || !cu_tokens || !entry_of_token)))
+    return SHARPI_ERR_ARG;
+  if (norm_mode < 0 || norm_mode > 2 || (norm_mode && (!q_norm_w || !k_norm_w))) return SHARPI_ERR_ARG;
+  if (rotary_dim < 0 || rotary_dim % 2 || rotary_dim > hd || (rotary_dim > 0 && !inv_freq)) return SHARPI_ERR_ARG;
+  if (v_off < 0 && vd != hd) return SHARPI_ERR_ARG;
+  if (slot_mapping && (!k_cache || !v_cache || page_size <= 0)) return SHARPI_ERR_ARG;
+  const int qn = nh * hd, kn = nkv * hd, vn = v_off >= 0 ? nkv * vd : 0;
+  const size_t lds = (size_t)(qn + kn + vn) * sizeof(float);
+  if (lds > 60 * 1024) return SHARPI_ERR_ARG;
+  PrepArgs a{proj, stride, q_off, k_off, v_off, nh, nkv, hd, vd, conv_w, taps, tail, state_slots, entry_of_token,
+             cu_tokens, positions, norm_mode, q_norm_w, k_norm_w, eps, rotary_dim > 0 ? inv_freq : nullptr, rotary_dim,
+             half_split, magnitude, q_out, k_cache, v_cache, slot_mapping, page_size};
+  if (dtype == DT_F32) qk_prep_kernel<float><<<n_tokens, kPrepThreads, lds, stream>>>(a);
+  else if (dtype == DT_BF16) qk_prep_kernel<bf16_t><<<n_tokens, kPrepThreads, lds, stream>>>(a);
+  else return SHARPI_ERR_ARG;
+  SHARPI_CHECK_LAUNCH();
+  if (taps > 0 && update_tail) {
+    dim3 grid(ceil_div(qn + kn + vn, 256), n_entries);
+    if (dtype == DT_F32)
+      conv_tail_kernel<float><<<grid, 256, 0, stream>>>((const float*)proj, stride, q_off, k_off, v_off, qn, kn, vn, taps,
+                                                        tail, state_slots, cu_tokens);
+    else
+      conv_tail_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)proj, stride, q_off, k_off, v_off, qn, kn, vn, taps,
+                                                         tail, state_slots, cu_tokens);
+    SHARPI_CHECK_LAUNCH();
+  }
+  return SHARPI_OK;
+}

@@ -16,7 +16,7 @@ from typing import Callable, Dict, Hashable, Iterator, List, Optional, Sequence,
 import torch
 
 from ..cache.manager import CacheManager, pool_sizes
-from ..cache.spec import KVSpec
+from ..cache.spec import kv_of
 from ..config.base import ModelConfig, load_config
 from ..registry import build_model
 from ..sampling.params import SamplingParams
@@ -101,10 +101,11 @@ class Engine:
             self.config.validate()
         else:
             raise ValueError("give a model folder or a configuration")
-        self.model = build_model(self.config)
         if model_dir is not None:
             source = SafetensorsSource(model_dir, self.dtype, self.device)
-        else:
+            self.config = self.config.with_tensor_shapes(source.available())
+        self.model = build_model(self.config)
+        if model_dir is None:
             if weight_seed is None:
                 raise ValueError("a configuration without a model folder needs weight_seed (random weights)")
             source = RandomSource(self.model.param_specs(), weight_seed, self.dtype, self.device,
@@ -133,7 +134,7 @@ class Engine:
         # group without a window gets that many, a windowed group only what its windows can ever
         # hold at once (window + one step, per request), however long the requests grow.
         width = torch.empty(0, dtype=self.dtype).element_size()
-        kv_specs = [s for s in specs if isinstance(s, KVSpec)]
+        kv_specs = [kv_of(s) for s in specs if kv_of(s) is not None]
         full_len = (self.max_model_len + page_size - 1) // page_size * page_size
         sizes = pool_sizes(specs, page_size, self.max_num_seqs, full_len, self.max_tokens_per_step,
                            None if kv_tokens is None else max(1, (int(kv_tokens) + page_size - 1) // page_size))

@@ -190,7 +190,7 @@ class ModelRunner:
         for i in range(len(cache.slot_specs)):
             g = cache.group_of_slot[i]
             out.append(LayerCache(group=ctx.groups[g] if g >= 0 else None, k=cache.k[i], v=cache.v[i],
-                                  state=cache.state[i], write=True))
+                                  state=cache.state[i], write=True, states=cache.states[i]))
         return out
 
     # ------------------------------------------------------------------

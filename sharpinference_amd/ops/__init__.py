@@ -272,9 +272,12 @@ def rope_kv(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slo
 
 def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                       entry_of_token: torch.Tensor, positions: torch.Tensor, window_kind: int, window: int,
-                      scale: float, nh: int, nkv: int, hd: int, vd: Optional[int] = None) -> torch.Tensor:
+                      scale: float, nh: int, nkv: int, hd: int, vd: Optional[int] = None, softcap: float = 0.0,
+                      sink: bool = False) -> torch.Tensor:
     """Attention of every token of the batch over its request's pages; float arithmetic.  Values
-    (and so the output, [T, nh*vd]) may have another width than keys."""
+    (and so the output, [T, nh*vd]) may have another width than keys.  softcap > 0: scores become
+    softcap * tanh(score / softcap); sink: one more term exp(0), without a value, in the softmax's
+    denominator."""
     _dev(q, k_cache, v_cache, block_table, entry_of_token, positions)
     _i32(block_table, "block_table")
     _i32(entry_of_token, "entry_of_token")
@@ -289,7 +292,7 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     out = torch.empty(T, nh * vd, dtype=q.dtype, device=q.device)
     _run("sharpi_attention_generic", _ptr(q), _ptr(k_cache), _ptr(v_cache), _code(q.dtype), _ptr(block_table),
          _ptr(entry_of_token), _ptr(positions), _ptr(out), int(window_kind), int(window), float(scale), T, nh, nkv,
-         hd, vd, k_cache.shape[2], block_table.shape[1], k_cache.shape[0], _stream())
+         hd, vd, k_cache.shape[2], block_table.shape[1], k_cache.shape[0], float(softcap), 1 if sink else 0, _stream())
     return out
 
 
@@ -310,7 +313,7 @@ def decode_attention_ok(dtype: torch.dtype, hd: int) -> bool:
 def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                      entry_of_token: torch.Tensor, positions: torch.Tensor, token_list: Optional[torch.Tensor],
                      max_context: int, window_kind: int, window: int, scale: float, nh: int, nkv: int, hd: int,
-                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     out: Optional[torch.Tensor] = None, softcap: float = 0.0, sink: bool = False) -> torch.Tensor:
     """Split-K flash-decode for the listed tokens (all tokens if token_list is None), each a
     single query over its request's pages.  `max_context` bounds position + 1 of every token."""
     _dev(q, k_cache, v_cache, block_table, entry_of_token, positions, token_list, out)
@@ -334,7 +337,7 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     _run("sharpi_attention_decode", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(entry_of_token),
          _ptr(positions), _ptr(token_list), _ptr(part_o), _ptr(part_ml), _ptr(out), int(window_kind), int(window),
          float(scale), n_list, nh, nkv, hd, k_cache.shape[2], block_table.shape[1], k_cache.shape[0], max_splits,
-         _stream())
+         float(softcap), 1 if sink else 0, _stream())
     return out
 
 
@@ -348,7 +351,7 @@ def prefill_attention_ok(dtype: torch.dtype, hd: int) -> bool:
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                       positions: torch.Tensor, tiles: torch.Tensor, window_kind: int, window: int, scale: float,
                       nh: int, nkv: int, hd: int, out: Optional[torch.Tensor] = None,
-                      tile_tokens: int = PREFILL_TILE_TOKENS) -> torch.Tensor:
+                      tile_tokens: int = PREFILL_TILE_TOKENS, softcap: float = 0.0, sink: bool = False) -> torch.Tensor:
     """Flash attention for the listed tiles: tiles int32 [n, 3] = (entry, first token, rows <=
     tile_tokens), the tokens of a tile consecutive in one entry.  tile_tokens (128, or 64: blocks of
     half the rows, for short prompts) is what the caller cut the tiles to; a row's result does not
@@ -369,7 +372,7 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _need(out.shape == q.shape and out.dtype == q.dtype, "attention_prefill: out must match q")
     _run("sharpi_attention_prefill", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(positions),
          _ptr(tiles), _ptr(out), tiles.shape[0], int(tile_tokens), int(window_kind), int(window), float(scale), nh,
-         nkv, hd, k_cache.shape[2], block_table.shape[1], k_cache.shape[0], _stream())
+         nkv, hd, k_cache.shape[2], block_table.shape[1], k_cache.shape[0], float(softcap), 1 if sink else 0, _stream())
     return out
 
 
@@ -1114,25 +1117,179 @@ def edit_logits(logits: torch.Tensor, row_offsets: torch.Tensor, ids: torch.Tens
 
 
 # ---------------------------------------------------------------------------
+# between the projections and attention, for layers that norm before they rotate
+# ---------------------------------------------------------------------------
+NORM_NONE, NORM_PER_HEAD, NORM_WHOLE = 0, 1, 2
+QK_PREP_MAX_TAPS = 8          # csrc/qk_prep.hip kPrepMaxTaps
+QK_PREP_MAX_ROW = 15 * 1024   # q + k + v channels of a token that the kernel holds in LDS as floats
+
+
+def qk_prep(proj: torch.Tensor, q_off: int, k_off: int, v_off: Optional[int], nh: int, nkv: int, hd: int, vd: int,
+            ctx, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor],
+            norm_mode: int = NORM_NONE, q_norm_w: Optional[torch.Tensor] = None, k_norm_w: Optional[torch.Tensor] = None,
+            eps: float = 1e-6, inv_freq: Optional[torch.Tensor] = None, pair_layout: int = PAIRS_INTERLEAVED,
+            magnitude: float = 1.0, conv_w: Optional[torch.Tensor] = None, tail: Optional[torch.Tensor] = None,
+            update_tail: bool = True) -> torch.Tensor:
+    """From a step's projections proj [T, N] (q at columns q_off.., k at k_off.., v at v_off.., or
+    v_off None: the values are the keys before norm and rotation): optional short causal
+    convolution over time on every channel (conv_w float32 [channels, taps]; tail float32 [slots,
+    taps - 1, channels] carries each request's last projected rows from step to step and is brought
+    up to date unless update_tail is False), RMS norm of q and k with learned weights (per head, or
+    over the whole projection), rotary positions (cos and sin times `magnitude`), keys and values
+    into the cache at slot_mapping (None: nothing is stored).  Returns q [T, nh*hd]."""
+    _dev(proj, k_cache, v_cache, slot_mapping, q_norm_w, k_norm_w, inv_freq, conv_w, tail)
+    _i32(slot_mapping, "slot_mapping")
+    T, N = proj.shape
+    own_v = v_off is not None
+    qn, kn, vn = nh * hd, nkv * hd, (nkv * vd if own_v else 0)
+    _need(proj.dim() == 2 and 0 <= q_off and q_off + qn <= N and 0 <= k_off and k_off + kn <= N
+          and (not own_v or (0 <= v_off and v_off + vn <= N)), "qk_prep: q, k and v columns must lie inside proj")
+    _need(own_v or vd == hd, "qk_prep: values taken from the keys have the keys' width")
+    _need(hd % 2 == 0 and qn + kn + vn <= QK_PREP_MAX_ROW, f"qk_prep: an even head size and at most {QK_PREP_MAX_ROW} channels a token")
+    _need(ctx.positions.shape == (T,), "qk_prep: the step's positions must be [T]")
+    if slot_mapping is not None:
+        _need(slot_mapping.shape == (T,) and _cache_shapes_ok(k_cache, v_cache, nkv, hd, vd) and k_cache.dtype == proj.dtype
+              and v_cache.dtype == proj.dtype, "qk_prep: slot_mapping [T]; caches K [pages, nkv, page_size, hd], V [pages, nkv, vd, page_size] of proj's dtype")
+    _need(norm_mode in (NORM_NONE, NORM_PER_HEAD, NORM_WHOLE), "qk_prep: norm_mode 0, 1 or 2")
+    if norm_mode != NORM_NONE:
+        want_q, want_k = ((hd,), (hd,)) if norm_mode == NORM_PER_HEAD else ((qn,), (kn,))
+        _need(q_norm_w is not None and k_norm_w is not None and q_norm_w.dtype == torch.float32 and k_norm_w.dtype == torch.float32
+              and tuple(q_norm_w.shape) == want_q and tuple(k_norm_w.shape) == want_k,
+              f"qk_prep: norm weights must be float32 {want_q} and {want_k}")
+    rotary_dim = 0
+    if inv_freq is not None:
+        _need(inv_freq.dtype == torch.float32 and inv_freq.dim() == 1 and 1 <= inv_freq.shape[0] <= hd // 2,
+              "qk_prep: inv_freq must be float32 [rotary_dim / 2], rotary_dim <= hd")
+        rotary_dim = 2 * inv_freq.shape[0]
+    taps = 0
+    if conv_w is not None:
+        taps = conv_w.shape[1]
+        _need(conv_w.dtype == torch.float32 and conv_w.shape == (qn + kn + vn, taps) and 2 <= taps <= QK_PREP_MAX_TAPS,
+              f"qk_prep: conv_w must be float32 [q + k + v channels, 2..{QK_PREP_MAX_TAPS} taps]")
+        _need(tail is not None and tail.dtype == torch.float32 and tail.dim() == 3 and tuple(tail.shape[1:]) == (taps - 1, qn + kn + vn),
+              "qk_prep: tail must be float32 [slots, taps - 1, channels]")
+        _need(ctx.state_slots.shape == (ctx.n_entries,) and ctx.cu_tokens.shape == (ctx.n_entries + 1,)
+              and ctx.entry_of_token.shape == (T,), "qk_prep: the step's per-entry arrays do not fit")
+    q_out = torch.empty(T, qn, dtype=proj.dtype, device=proj.device)
+    page_size = k_cache.shape[2] if k_cache is not None else 0
+    _run("sharpi_qk_prep", _ptr(proj), _code(proj.dtype), N, int(q_off), int(k_off), int(v_off) if own_v else -1, T,
+         ctx.n_entries, nh, nkv, hd, vd, _ptr(conv_w), taps, _ptr(tail), _ptr(ctx.state_slots), _ptr(ctx.entry_of_token),
+         _ptr(ctx.cu_tokens), _ptr(ctx.positions), int(norm_mode), _ptr(q_norm_w), _ptr(k_norm_w), float(eps),
+         _ptr(inv_freq), rotary_dim, 1 if pair_layout == PAIRS_HALF_SPLIT else 0, float(magnitude), _ptr(q_out),
+         _ptr(k_cache), _ptr(v_cache), _ptr(slot_mapping), page_size, 1 if update_tail else 0, _stream())
+    return q_out
+
+
+# ---------------------------------------------------------------------------
+# gated linear attention
+# ---------------------------------------------------------------------------
+GLA_MAX_KEY_DIM = 256      # key channels of a head that the walk holds (csrc/linear_attention.hip)
+
+
+def gla_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Tensor, z_bias: torch.Tensor, tau: float,
+             q_scale: float, state: torch.Tensor, ctx, nh: int, dk: int, dv: int) -> torch.Tensor:
+    """The recurrence S_t = diag(alpha_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per head, token by
+    token along every entry of the step, from and into state [slots, nh, dk, dv] (float32) at the
+    entries' state slots.  q, k (nh*dk columns each) and v (nh*dv) are columns of proj [T, N]; q is
+    multiplied by q_scale; alpha = sigmoid(z + z_bias)^(1/tau) with z float32 [T, nh*dk].  Returns
+    o float32 [T, nh*dv]."""
+    _dev(proj, z, z_bias, state)
+    T, N = proj.shape
+    _need(1 <= dk <= GLA_MAX_KEY_DIM and dv >= 1 and nh >= 1, f"gla_walk: key channels 1..{GLA_MAX_KEY_DIM}")
+    _need(min(q_off, k_off, v_off) >= 0 and max(q_off, k_off) + nh * dk <= N and v_off + nh * dv <= N,
+          "gla_walk: q, k and v columns must lie inside proj")
+    _need(z.dtype == torch.float32 and z.shape == (T, nh * dk) and z_bias.dtype == torch.float32 and z_bias.shape == (nh * dk,),
+          "gla_walk: z float32 [T, nh*dk] and z_bias float32 [nh*dk] wanted")
+    _need(state.dtype == torch.float32 and state.dim() == 4 and tuple(state.shape[1:]) == (nh, dk, dv),
+          "gla_walk: state must be float32 [slots, nh, dk, dv]")
+    _need(ctx.state_slots.shape == (ctx.n_entries,) and ctx.cu_tokens.shape == (ctx.n_entries + 1,) and ctx.n_tokens == T,
+          "gla_walk: the step's per-entry arrays do not fit")
+    out = torch.empty(T, nh * dv, dtype=torch.float32, device=proj.device)
+    _run("sharpi_gla_walk", _ptr(proj), _code(proj.dtype), N, int(q_off), int(k_off), int(v_off), _ptr(z), _ptr(z_bias),
+         float(tau), float(q_scale), _ptr(state), _ptr(ctx.state_slots), _ptr(ctx.cu_tokens), _ptr(out), ctx.n_entries,
+         nh, dk, dv, _stream())
+    return out
+
+
+def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, eps: float, nh: int, dv: int, out_dtype: torch.dtype,
+                   gate_proj: Optional[torch.Tensor] = None, gate_off: int = 0) -> torch.Tensor:
+    """o float32 [T, nh*dv] -> per (token, head) unit RMS over dv, times weight [dv] (shared by the
+    heads), times silu of the gate (columns gate_off.. of gate_proj [T, N], of out_dtype; None: no gate)."""
+    _dev(o, weight, gate_proj)
+    T = o.shape[0]
+    _need(o.dtype == torch.float32 and o.shape == (T, nh * dv) and weight.dtype == torch.float32 and weight.shape == (dv,),
+          "head_norm_gate: o float32 [T, nh*dv], weight float32 [dv]")
+    stride = 0
+    if gate_proj is not None:
+        _need(gate_proj.dtype == out_dtype and gate_proj.dim() == 2 and gate_proj.shape[0] == T
+              and 0 <= gate_off and gate_off + nh * dv <= gate_proj.shape[1], "head_norm_gate: the gate's columns must lie inside gate_proj")
+        stride = gate_proj.shape[1]
+    out = torch.empty(T, nh * dv, dtype=out_dtype, device=o.device)
+    _run("sharpi_head_norm_gate", _ptr(o), _ptr(weight), float(eps), _ptr(gate_proj), _code(out_dtype), stride, int(gate_off),
+         _ptr(out), T, nh, dv, _stream())
+    return out
+
+
+UNGATED_ACTIVATIONS = {"relu2": 1, "gelu_tanh": 2, "silu": 3}
+
+
+def activation(x: torch.Tensor, name: str) -> torch.Tensor:
+    """f(x) element by element, f one of UNGATED_ACTIVATIONS (relu2: the square of relu)."""
+    _dev(x)
+    _need(name in UNGATED_ACTIVATIONS, f"activation {name!r} is not known ({', '.join(sorted(UNGATED_ACTIVATIONS))})")
+    out = torch.empty_like(x)
+    _run("sharpi_activation", _ptr(x), _ptr(out), _code(x.dtype), x.numel(), UNGATED_ACTIVATIONS[name], _stream())
+    return out
+
+
+NORM_MEAN_MAX_BRANCHES = 4
+
+
+def norm_mean(xs, weights, eps: float) -> torch.Tensor:
+    """The mean over branches b of unit_rms(xs[b]) * weights[b], row by row: xs tensors [T, N] of one
+    dtype, weights float32 [N].  Returns float32 [T, N]."""
+    import ctypes
+
+    n = len(xs)
+    _need(1 <= n <= NORM_MEAN_MAX_BRANCHES and len(weights) == n, f"norm_mean: 1 to {NORM_MEAN_MAX_BRANCHES} branches, a weight vector each")
+    _dev(*xs, *weights)
+    T, N = xs[0].shape
+    for x, w in zip(xs, weights):
+        _need(x.shape == (T, N) and x.dtype == xs[0].dtype and w.dtype == torch.float32 and w.shape == (N,),
+              "norm_mean: branches [T, N] of one dtype, weights float32 [N]")
+    out = torch.empty(T, N, dtype=torch.float32, device=xs[0].device)
+    xp = (ctypes.c_void_p * n)(*[x.data_ptr() for x in xs])
+    wp = (ctypes.c_void_p * n)(*[w.data_ptr() for w in weights])
+    _run("sharpi_norm_mean", ctypes.cast(xp, ctypes.c_void_p), ctypes.cast(wp, ctypes.c_void_p), n, _code(xs[0].dtype),
+         _ptr(out), T, N, float(eps), _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------
 # dispatchers used by the parts
 # ---------------------------------------------------------------------------
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, group, ctx, window_kind: int,
-              window: int, scale: float, nh: int, nkv: int, hd: int, vd: Optional[int] = None) -> torch.Tensor:
+              window: int, scale: float, nh: int, nkv: int, hd: int, vd: Optional[int] = None, softcap: float = 0.0,
+              sink: bool = False) -> torch.Tensor:
     """Attention of the step's tokens over their requests' pages (`group`: the cache group's
-    block tables, `ctx`: the step).  Values of another width than keys (vd) go through the float kernel."""
+    block tables, `ctx`: the step).  Values of another width than keys (vd) go through the float kernel.
+    softcap > 0 caps the scores (softcap * tanh(score / softcap)); sink adds a key of score 0 without a
+    value to the softmax's denominator."""
     same = vd is None or vd == hd
     if same and decode_attention_ok(q.dtype, hd) and (prefill_attention_ok(q.dtype, hd) or not ctx.n_prefill_tiles):
         # entries of one token: split-K decode kernel; longer entries: flash kernel, a tile of tokens a block
         out = torch.empty_like(q)
         if ctx.n_prefill_tiles:
             attention_prefill(q, k_cache, v_cache, group.block_table, ctx.positions, ctx.prefill_tiles, window_kind,
-                              window, scale, nh, nkv, hd, out=out, tile_tokens=ctx.prefill_tile_tokens)
+                              window, scale, nh, nkv, hd, out=out, tile_tokens=ctx.prefill_tile_tokens, softcap=softcap,
+                              sink=sink)
         if ctx.n_decode:
             attention_decode(q, k_cache, v_cache, group.block_table, ctx.entry_of_token, ctx.positions,
-                             ctx.decode_tokens, group.max_context, window_kind, window, scale, nh, nkv, hd, out=out)
+                             ctx.decode_tokens, group.max_context, window_kind, window, scale, nh, nkv, hd, out=out,
+                             softcap=softcap, sink=sink)
         return out
     return attention_generic(q, k_cache, v_cache, group.block_table, ctx.entry_of_token, ctx.positions, window_kind,
-                             window, scale, nh, nkv, hd, vd)
+                             window, scale, nh, nkv, hd, vd, softcap=softcap, sink=sink)
 
 
 def grouped_swiglu(x: torch.Tensor, w_gate_up, rt: Routing, out_dtype: torch.dtype, scaled: bool = True,

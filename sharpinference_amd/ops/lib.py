@@ -28,9 +28,9 @@ _SIGNATURES = {
     "sharpi_peak_mfma": [P, I, I, P],
     "sharpi_random_fill": [P, I, c_longlong, c_ulonglong, I, F, I, I, P],
     "sharpi_rope_kv": [P, P, P, P, I, P, P, P, P, I, F, I, F, F, I, I, I, I, I, I, I, I, P],
-    "sharpi_attention_generic": [P, P, P, I, P, P, P, P, I, I, F, I, I, I, I, I, I, I, I, P],
-    "sharpi_attention_decode": [P, P, P, P, P, P, P, P, P, P, I, I, F, I, I, I, I, I, I, I, I, P],
-    "sharpi_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, F, I, I, I, I, I, I, P],
+    "sharpi_attention_generic": [P, P, P, I, P, P, P, P, I, I, F, I, I, I, I, I, I, I, I, F, I, P],
+    "sharpi_attention_decode": [P, P, P, P, P, P, P, P, P, P, I, I, F, I, I, I, I, I, I, I, I, F, I, P],
+    "sharpi_attention_prefill": [P, P, P, P, P, P, P, I, I, I, I, F, I, I, I, I, I, I, F, I, P],
     "sharpi_gemm_tiled": [P, P, P, I, I, I, I, I, P, P, I, P],
     "sharpi_gemm_skinny": [P, P, P, I, I, I, I, P, P, I, I, I, I, I, P],
     "sharpi_gemm_skinny_swiglu": [P, P, P, I, I, I, P, P, I, P, I, I, I, I, I, P],
@@ -49,6 +49,11 @@ _SIGNATURES = {
     "sharpi_argmax_rows": [P, P, I, I, P],
     "sharpi_sample_rows": [P, P, P, P, P, P, P, P, I, I, P],
     "sharpi_edit_logits": [P, P, P, P, P, P, P, P, I, I, P],
+    "sharpi_qk_prep": [P, I, I, I, I, I, I, I, I, I, I, I, P, I, P, P, P, P, P, I, P, P, F, P, I, I, F, P, P, P, P, I, I, P],
+    "sharpi_gla_walk": [P, I, I, I, I, I, P, P, F, F, P, P, P, P, I, I, I, I, P],
+    "sharpi_head_norm_gate": [P, P, F, P, I, I, I, P, I, I, I, P],
+    "sharpi_activation": [P, P, I, c_longlong, I, P],
+    "sharpi_norm_mean": [P, P, I, I, P, I, I, F, P],
 }
 
 # entry points that newer sources add; bound when present

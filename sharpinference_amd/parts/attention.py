@@ -10,8 +10,8 @@ import torch
 from .. import ops
 from ..ops.lib import PREFILL_TILE_TOKENS
 from ..ops.profile import section
-from ..cache.spec import KVSpec, WINDOW_CHUNK, WINDOW_NONE, WINDOW_SLIDING  # noqa: F401
-from .base import HostStep, LayerCache, ParamSpec, Part, StepContext, StepPlanner, TensorSource
+from ..cache.spec import KVSpec, MixedSpec, StateSpec, kv_of, WINDOW_CHUNK, WINDOW_NONE, WINDOW_SLIDING  # noqa: F401
+from .base import INIT_NORM_WEIGHT, HostStep, LayerCache, ParamSpec, Part, StepContext, StepPlanner, TensorSource
 
 SHORT_PROMPT_TOKENS = 1536   # up to so many prompt tokens in a step, tiles of half as many tokens (measured:
                              # 20-25 % less attention time from 512 to 1,536 tokens, 6 % more at 2,048)
@@ -62,16 +62,40 @@ class Attention(Part):
     ``head_dim``, see parts/position.py), ``v_head_dim`` (values and a head's output of another width than
     keys: such layers run the float attention kernel), ``qk_norm_eps`` (None = no norm), ``q_temperature`` = (floor_scale, attn_scale)
     multiplying queries by 1 + attn_scale * ln(floor((pos + 1) / floor_scale) + 1), and the
-    window: all keys, the chunk [floor(pos/W)*W, pos], or the last W keys."""
+    window: all keys, the chunk [floor(pos/W)*W, pos], or the last W keys.
+
+    Further options, for designs that norm before they rotate (they take the other kernel between
+    the projections and attention, csrc/qk_prep.hip):
+    ``qk_norm_weights``: "head" (an RMS norm of every query and key head with learned weights [head_dim]
+    shared by the heads) or "projection" (one RMS norm over all of a token's query heads, and one
+    over all its key heads, weights [heads * head_dim]); eps is ``qk_norm_eps``; the norm comes
+    BEFORE the rotation.  ``values_from_keys``: no value projection; a value is its key as
+    projected, before norm and rotation.  ``conv_taps`` n >= 2: a causal convolution over time on
+    every channel of q, k and v right behind the projections, y_t = sum_j w[:, j] u_(t - n + 1 + j)
+    (weights [channels, n]; zeros before a sequence's start; the last n - 1 projected rows of a
+    request are carried in its state slot).  ``softcap`` c: scores become c tanh(score / c).
+    ``sink``: the softmax's denominator holds one more term exp(0), a key of score 0 that has no
+    value.  A rotary object's ``magnitude`` multiplies cos and sin.  ``names``: the tensors' names
+    behind the layer's prefix."""
+
+    NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+             "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias",
+             "q_norm": "q_norm.weight", "k_norm": "k_norm.weight",
+             "q_conv": "q_conv.weight", "k_conv": "k_conv.weight", "v_conv": "v_conv.weight"}
 
     def __init__(self, hidden: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  rotary=None, qk_norm_eps: Optional[float] = None,
                  q_temperature: Optional[Tuple[float, float]] = None, window_kind: int = WINDOW_NONE,
                  window: int = 0, scale: Optional[float] = None, bias: bool = False, o_bias: Optional[bool] = None,
-                 v_head_dim: Optional[int] = None):
+                 v_head_dim: Optional[int] = None, qk_norm_weights: Optional[str] = None, values_from_keys: bool = False,
+                 conv_taps: int = 0, softcap: float = 0.0, sink: bool = False, names: Optional[Dict[str, str]] = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads cannot share {num_kv_heads} kv heads")
-        if head_dim % 16 or not 16 <= head_dim <= 256:
+        prep = bool(qk_norm_weights or values_from_keys or conv_taps)
+        if prep:
+            if head_dim % 2 or not 2 <= head_dim <= 256:
+                raise ValueError(f"head_dim {head_dim} is not taken: even sizes from 2 to 256")
+        elif head_dim % 16 or not 16 <= head_dim <= 256:
             raise ValueError(f"head_dim {head_dim} is not taken: multiples of 16 from 16 to 256")
         if rotary is not None and rotary.head_dim != head_dim:
             raise ValueError("the rotary table's head_dim differs from the mixer's")
@@ -86,49 +110,99 @@ class Attention(Part):
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
         self.bias = bool(bias)                                   # q, k and v carry biases
         self.o_bias = self.bias if o_bias is None else bool(o_bias)   # the output projection carries one
+        if qk_norm_weights not in (None, "head", "projection"):
+            raise ValueError(f"qk_norm_weights {qk_norm_weights!r} is not known (None, 'head', 'projection')")
+        if qk_norm_weights and qk_norm_eps is None:
+            raise ValueError("a norm with weights needs qk_norm_eps")
+        if values_from_keys and self.vd != self.hd:
+            raise ValueError("values taken from the keys have the keys' width")
+        self.conv_taps = int(conv_taps)
+        if self.conv_taps and not 2 <= self.conv_taps <= ops.QK_PREP_MAX_TAPS:
+            raise ValueError(f"a convolution of {conv_taps} taps is not taken: 2 to {ops.QK_PREP_MAX_TAPS}")
+        self.qk_norm_weights, self.values_from_keys = qk_norm_weights, bool(values_from_keys)
+        self.softcap, self.sink = float(softcap or 0.0), bool(sink)
+        if self.softcap < 0:
+            raise ValueError("softcap must be positive (or 0 for none)")
+        self.prep = prep                                         # the layer takes the norm-before-rotation kernel
+        if prep and (q_temperature is not None or bias):
+            raise ValueError("query temperature and q/k/v biases belong to the rotate-then-norm form of the layer")
+        if prep and (self.nh + 2 * self.nkv) * max(self.hd, self.vd) > ops.QK_PREP_MAX_ROW:
+            raise ValueError(f"a token's q, k and v of more than {ops.QK_PREP_MAX_ROW} channels are not taken")
+        if not prep and rotary is not None and getattr(rotary, "magnitude", 1.0) != 1.0:
+            raise ValueError("a rotation with a magnitude belongs to the norm-before-rotation form of the layer")
+        self.graph_safe = True                                   # its state (a convolution's tail) is walked on the device
+        self.names = {**self.NAMES, **(names or {})}
         self.w_qkv: Optional[torch.Tensor] = None
         self.w_o: Optional[torch.Tensor] = None
         self.b_qkv: Optional[torch.Tensor] = None                # float32 [q + 2 kv]: added by the rotation kernel
         self.b_o: Optional[torch.Tensor] = None                  # float32 [hidden]
+        self.w_q_norm: Optional[torch.Tensor] = None             # float32
+        self.w_k_norm: Optional[torch.Tensor] = None
+        self.w_conv: Optional[torch.Tensor] = None               # float32 [q + k + v channels, taps]
 
     # -- what it needs --------------------------------------------------------
     def step_planners(self):
         return (_WORK_LISTS,)
 
-    def cache_spec(self) -> KVSpec:
-        return KVSpec(self.nkv, self.hd, self.window_kind, self.window, 0 if self.vd == self.hd else self.vd)
+    @property
+    def _channels(self) -> int:
+        """Projected channels of a token: q, k and (where the layer has a value projection) v."""
+        return self.nh * self.hd + self.nkv * self.hd + (0 if self.values_from_keys else self.nkv * self.vd)
+
+    def cache_spec(self):
+        kv = KVSpec(self.nkv, self.hd, self.window_kind, self.window, 0 if self.vd == self.hd else self.vd)
+        if not self.conv_taps:
+            return kv
+        return MixedSpec(kv, (StateSpec((self.conv_taps - 1, self._channels), torch.float32),))
 
     def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
         q, kv, vv, ov = self.nh * self.hd, self.nkv * self.hd, self.nkv * self.vd, self.nh * self.vd
+        n = self.names
         specs = {
-            prefix + "q_proj.weight": ParamSpec((q, self.hidden)),
-            prefix + "k_proj.weight": ParamSpec((kv, self.hidden)),
-            prefix + "v_proj.weight": ParamSpec((vv, self.hidden)),
-            prefix + "o_proj.weight": ParamSpec((self.hidden, ov)),
+            prefix + n["q"]: ParamSpec((q, self.hidden)),
+            prefix + n["k"]: ParamSpec((kv, self.hidden)),
+            prefix + n["o"]: ParamSpec((self.hidden, ov)),
         }
+        if not self.values_from_keys:
+            specs[prefix + n["v"]] = ParamSpec((vv, self.hidden))
         if self.bias:
-            specs.update({prefix + "q_proj.bias": ParamSpec((q,)), prefix + "k_proj.bias": ParamSpec((kv,)),
-                          prefix + "v_proj.bias": ParamSpec((vv,))})
+            specs.update({prefix + n["q_bias"]: ParamSpec((q,)), prefix + n["k_bias"]: ParamSpec((kv,)),
+                          prefix + n["v_bias"]: ParamSpec((vv,))})
         if self.o_bias:
-            specs[prefix + "o_proj.bias"] = ParamSpec((self.hidden,))
+            specs[prefix + n["o_bias"]] = ParamSpec((self.hidden,))
+        if self.qk_norm_weights:
+            whole = self.qk_norm_weights == "projection"
+            specs[prefix + n["q_norm"]] = ParamSpec((q if whole else self.hd,), INIT_NORM_WEIGHT)
+            specs[prefix + n["k_norm"]] = ParamSpec((kv if whole else self.hd,), INIT_NORM_WEIGHT)
+        if self.conv_taps:
+            specs[prefix + n["q_conv"]] = ParamSpec((q, self.conv_taps))
+            specs[prefix + n["k_conv"]] = ParamSpec((kv, self.conv_taps))
+            if not self.values_from_keys:
+                specs[prefix + n["v_conv"]] = ParamSpec((vv, self.conv_taps))
         return specs
 
     def load(self, prefix: str, source: TensorSource) -> None:
-        q, kv, vv = self.nh * self.hd, self.nkv * self.hd, self.nkv * self.vd
-        parts = [source.get(prefix + n + "_proj.weight") for n in ("q", "k", "v")]
+        n = self.names
+        kinds = ("q", "k") if self.values_from_keys else ("q", "k", "v")
+        parts = [source.get(prefix + n[k]) for k in kinds]
         dt = torch.float32 if any(p.dtype == torch.float32 for p in parts) else parts[0].dtype
-        fused = torch.empty(q + kv + vv, self.hidden, dtype=dt, device=parts[0].device)
+        fused = torch.empty(sum(p.shape[0] for p in parts), self.hidden, dtype=dt, device=parts[0].device)
         o = 0
         for p in parts:
             fused[o:o + p.shape[0]].copy_(p)
             o += p.shape[0]
         # both also in the order the few-rows kernel streams them; the rows stay for prompt-sized steps
         self.w_qkv = ops.pack_weight(fused)
-        self.w_o = ops.pack_weight(source.get(prefix + "o_proj.weight"))
+        self.w_o = ops.pack_weight(source.get(prefix + n["o"]))
         if self.bias:
-            self.b_qkv = torch.cat([source.get(prefix + n + "_proj.bias").float() for n in ("q", "k", "v")]).contiguous()
+            self.b_qkv = torch.cat([source.get(prefix + n[k + "_bias"]).float() for k in ("q", "k", "v")]).contiguous()
         if self.o_bias:
-            self.b_o = source.get(prefix + "o_proj.bias").float().contiguous()
+            self.b_o = source.get(prefix + n["o_bias"]).float().contiguous()
+        if self.qk_norm_weights:
+            self.w_q_norm = source.get(prefix + n["q_norm"]).float().contiguous()
+            self.w_k_norm = source.get(prefix + n["k_norm"]).float().contiguous()
+        if self.conv_taps:
+            self.w_conv = torch.cat([source.get(prefix + n[k + "_conv"]).float() for k in kinds]).contiguous()
 
     # -- compute --------------------------------------------------------------
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
@@ -143,23 +217,32 @@ class Attention(Part):
         inv_freq = self.rotary.table(x.device) if self.rotary is not None else None
         layout = ops.PAIRS_HALF_SPLIT if self.rotary is not None and self.rotary.pair_layout == "half" else ops.PAIRS_INTERLEAVED
         with section("rope + cache write", nbytes=2 * width * T * (q_dim + 2 * kv_dim)):
-            q = ops.rope_kv(qkv, cache.k, cache.v, slots, ctx.positions, inv_freq, self.qk_norm_eps is not None,
-                            self.qk_norm_eps or 1e-6, self.q_temperature, self.nh, self.nkv, self.hd, layout,
-                            bias=self.b_qkv, vd=self.vd)
+            if self.prep:
+                mode = {None: ops.NORM_NONE, "head": ops.NORM_PER_HEAD, "projection": ops.NORM_WHOLE}[self.qk_norm_weights]
+                kn = self.nkv * self.hd
+                q = ops.qk_prep(qkv, 0, q_dim, None if self.values_from_keys else q_dim + kn, self.nh, self.nkv, self.hd,
+                                self.vd, ctx, cache.k, cache.v, slots, mode, self.w_q_norm, self.w_k_norm,
+                                self.qk_norm_eps or 1e-6, inv_freq, layout,
+                                getattr(self.rotary, "magnitude", 1.0) if self.rotary is not None else 1.0,
+                                self.w_conv, cache.states[0] if self.conv_taps else None, update_tail=cache.write)
+            else:
+                q = ops.rope_kv(qkv, cache.k, cache.v, slots, ctx.positions, inv_freq, self.qk_norm_eps is not None,
+                                self.qk_norm_eps or 1e-6, self.q_temperature, self.nh, self.nkv, self.hd, layout,
+                                bias=self.b_qkv, vd=self.vd)
         with section("attention", nbytes=lambda: self._keys_held(ctx) * 2 * kv_dim * width + 2 * T * q_dim * width,
                      flops=lambda: 4.0 * self._keys_read(ctx) * q_dim):
             o = ops.attention(q, cache.k, cache.v, g, ctx, self.window_kind, self.window, self.scale, self.nh, self.nkv,
-                              self.hd, self.vd)
+                              self.hd, self.vd, softcap=self.softcap, sink=self.sink)
         with section("o", nbytes=width * self.hidden * (q_dim + T) + width * T * q_dim, flops=2.0 * T * self.hidden * q_dim):
             out = ops.linear(o, self.w_o, ctx.act_dtype)
             return ops.add_bias(out, self.b_o) if self.b_o is not None else out
 
     def _keys_read(self, ctx: StepContext) -> int:
         """(query, key) pairs of the step: what is computed."""
-        spec = self.cache_spec()
+        spec = kv_of(self.cache_spec())
         return sum(p - spec.first_visible(p) + 1 for s, n in zip(ctx.entry_starts, ctx.entry_lens) for p in range(s, s + n))
 
     def _keys_held(self, ctx: StepContext) -> int:
         """Keys that some query of the step sees, each counted once per entry: what has to be read."""
-        spec = self.cache_spec()
+        spec = kv_of(self.cache_spec())
         return sum(s + n - spec.first_visible(s) for s, n in zip(ctx.entry_starts, ctx.entry_lens))

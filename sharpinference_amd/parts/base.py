@@ -111,8 +111,9 @@ class LayerCache:
     group: Optional[GroupView] = None
     k: Optional[torch.Tensor] = None   # [pages, kv heads, page_size, head_dim]
     v: Optional[torch.Tensor] = None
-    state: Optional[torch.Tensor] = None   # [state slots, ...]
+    state: Optional[torch.Tensor] = None   # [state slots, ...]: the layer's (first) fixed-size state
     write: bool = True                 # False: read another layer's cache, store nothing
+    states: Sequence[torch.Tensor] = ()    # every fixed-size state the layer asked for, in its order
 
 
 class ResidualStream:

@@ -51,9 +51,9 @@ class PreNormBlock(Part):
     def decode_graph_safe(self) -> bool:
         """Can a decode step through this block be captured into a graph?  Paged attention can; a
         mixer with state of its own says so itself (``graph_safe``)."""
-        from ..cache.spec import StateSpec
+        from ..cache.spec import states_of
 
-        return not isinstance(self.cache_spec(), StateSpec) or bool(getattr(self.mixer, "graph_safe", False))
+        return not states_of(self.cache_spec()) or bool(getattr(self.mixer, "graph_safe", False))
 
     def forward(self, stream: ResidualStream, ctx: StepContext, cache: LayerCache) -> None:
         n = self.norm1.forward(stream, ctx.act_dtype)
@@ -97,3 +97,30 @@ class PostNormBlock(PreNormBlock):
         if self.ffn is not None:
             y = self.ffn.forward(stream.act, ctx)
             self.norm2.add_normed(stream, y, ctx.act_dtype)
+
+
+class SandwichBlock(PreNormBlock):
+    """h += norm1b(mixer(norm1(h))); h += norm2b(ffn(norm2(h))): a norm before and a norm after each
+    branch.  ``ffn`` None: a layer of a mixer alone.  Nothing is left pending: the norm behind a
+    branch adds into the float residual sum itself."""
+
+    def __init__(self, norm1: Part, mixer: Part, norm1b: Part, norm2: Part = None, ffn: Part = None, norm2b: Part = None,
+                 names=None):
+        if not ((norm2 is None) == (ffn is None) == (norm2b is None)):
+            raise ValueError("a feed-forward and its two norms come together")
+        super().__init__(norm1, mixer, norm2, ffn, names or {"norm1": "norm1.", "mixer": "mixer.", "norm1b": "norm1b.",
+                                                             "norm2": "norm2.", "ffn": "ffn.", "norm2b": "norm2b."})
+        self.norm1b, self.norm2b = norm1b, norm2b
+
+    def _children(self):
+        kids = [(self.names["norm1"], self.norm1), (self.names["mixer"], self.mixer), (self.names["norm1b"], self.norm1b)]
+        if self.ffn is not None:
+            kids += [(self.names["norm2"], self.norm2), (self.names["ffn"], self.ffn), (self.names["norm2b"], self.norm2b)]
+        return tuple(kids)
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: LayerCache) -> None:
+        n = self.norm1.forward(stream, ctx.act_dtype)           # (folds in what a block before may have left pending)
+        self.norm1b.add_normed(stream, self.mixer.forward(n, ctx, cache), None)
+        if self.ffn is not None:
+            n = self.norm2.forward(stream, ctx.act_dtype)
+            self.norm2b.add_normed(stream, self.ffn.forward(n, ctx), None)

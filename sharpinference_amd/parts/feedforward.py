@@ -69,6 +69,35 @@ class DenseSwiGLU(Part):
             return ops.linear(act, self.w_down, ctx.act_dtype)
 
 
+class DenseMLP(Part):
+    """down( act(up x) ): a feed-forward without a gate.  ``activation``: "relu2" (the square of
+    relu), "gelu_tanh" or "silu".  ``names``: the two matrices' names behind the part's prefix."""
+
+    def __init__(self, hidden: int, intermediate: int, activation: str = "relu2", names: Optional[Dict[str, str]] = None):
+        if activation not in ops.UNGATED_ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not known ({', '.join(sorted(ops.UNGATED_ACTIVATIONS))})")
+        self.hidden, self.inter, self.activation = int(hidden), int(intermediate), activation
+        self.names = {"up": "up_proj.weight", "down": "down_proj.weight", **(names or {})}
+        self.w_up = None
+        self.w_down = None
+
+    def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
+        return {prefix + self.names["up"]: ParamSpec((self.inter, self.hidden)),
+                prefix + self.names["down"]: ParamSpec((self.hidden, self.inter))}
+
+    def load(self, prefix: str, source: TensorSource) -> None:
+        self.w_up = ops.pack_weight(source.get(prefix + self.names["up"]))
+        self.w_down = ops.pack_weight(source.get(prefix + self.names["down"]))
+
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        T = x.shape[0]
+        width = 2 if ctx.act_dtype == torch.bfloat16 else 4
+        with section("dense feed-forward", nbytes=width * 2 * self.inter * self.hidden + width * T * (2 * self.hidden + 3 * self.inter),
+                     flops=4.0 * T * self.inter * self.hidden):
+            up = ops.linear(x, self.w_up, ctx.act_dtype)
+            return ops.linear(ops.activation(up, self.activation), self.w_down, ctx.act_dtype)
+
+
 class MoESwiGLU(Part):
     """Router -> top-k experts (+ an always-on shared expert)
     (reference: src/SharpInference.Engine/ForwardPass.cs:2021-2098).

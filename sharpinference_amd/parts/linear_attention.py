@@ -1,0 +1,105 @@
+"""The gated linear attention mixer: a matrix-valued state per head instead of a cache of keys."""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from .. import ops
+from ..cache.spec import StateSpec
+from ..ops.profile import section
+from .base import INIT_NORM_WEIGHT, LayerCache, ParamSpec, Part, StepContext, TensorSource
+
+
+class GatedLinearAttention(Part):
+    """Linear attention with a decay per key channel.  With h the input, per head (dk key
+    channels, dv value channels): q = W_q h * dk^(-1/2), k = W_k h, v = W_v h, and a decay
+    alpha = sigmoid(z)^(1/tau) in (0, 1) for every key channel, z = W_a2 (W_a1 h) + b through a
+    narrow middle (``decay_rank``).  The state S [dk, dv] starts at zero and moves token by token,
+    S_t = diag(alpha_t) S_(t-1) + k_t v_t^T; the head's output is o_t = S_t^T q_t, RMS-normed over
+    dv with learned weights shared by the heads; the heads side by side are multiplied by
+    silu(W_g h) and projected by W_o.
+
+    What is kept per request is the state alone, [heads, dk, dv] in float, in the request's state
+    slot: no pages.  Decays (their logarithm, the division by tau, the exponential), the state and
+    the norm are float whatever the activations are stored as.  A step walks each entry's tokens
+    in order from the slot's state (csrc/linear_attention.hip), so the outputs of a token do not
+    depend on how its request was cut into steps."""
+
+    NAMES = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o", "norm": "norm", "a1": "a1", "a2": "a2", "a2_bias": "a2.b"}
+
+    def __init__(self, hidden: int, num_heads: int, key_dim: int, value_dim: int, tau: float, decay_rank: int,
+                 norm_eps: float, gate: bool = True, names: Optional[Dict[str, str]] = None):
+        if min(num_heads, key_dim, value_dim, decay_rank) < 1:
+            raise ValueError("heads, key_dim, value_dim and decay_rank must be positive")
+        if key_dim > ops.GLA_MAX_KEY_DIM:
+            raise ValueError(f"{key_dim} key channels a head are not taken: at most {ops.GLA_MAX_KEY_DIM}")
+        if not tau > 0:
+            raise ValueError("tau must be positive")
+        self.hidden, self.nh, self.dk, self.dv = int(hidden), int(num_heads), int(key_dim), int(value_dim)
+        self.tau, self.rank, self.eps, self.has_gate = float(tau), int(decay_rank), float(norm_eps), bool(gate)
+        self.names = {**self.NAMES, **(names or {})}
+        self.graph_safe = True         # entries and their state slots are read from the step's device arrays
+        self.w_in = None               # [q | k | v | g] rows: one product of the input
+        self.w_a1 = None
+        self.w_a2 = None
+        self.b_a2: Optional[torch.Tensor] = None      # float32 [heads * dk]
+        self.w_norm: Optional[torch.Tensor] = None    # float32 [dv]
+        self.w_o = None
+
+    def cache_spec(self) -> StateSpec:
+        return StateSpec((self.nh, self.dk, self.dv), torch.float32)
+
+    def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
+        n, qk, vv = self.names, self.nh * self.dk, self.nh * self.dv
+        specs = {
+            prefix + n["q"]: ParamSpec((qk, self.hidden)),
+            prefix + n["k"]: ParamSpec((qk, self.hidden)),
+            prefix + n["v"]: ParamSpec((vv, self.hidden)),
+            prefix + n["o"]: ParamSpec((self.hidden, vv)),
+            prefix + n["norm"]: ParamSpec((self.dv,), INIT_NORM_WEIGHT),
+            prefix + n["a1"]: ParamSpec((self.rank, self.hidden)),
+            prefix + n["a2"]: ParamSpec((qk, self.rank)),
+            prefix + n["a2_bias"]: ParamSpec((qk,)),
+        }
+        if self.has_gate:
+            specs[prefix + n["g"]] = ParamSpec((vv, self.hidden))
+        return specs
+
+    def load(self, prefix: str, source: TensorSource) -> None:
+        n = self.names
+        parts = [source.get(prefix + n[k]) for k in (("q", "k", "v", "g") if self.has_gate else ("q", "k", "v"))]
+        dt = torch.float32 if any(p.dtype == torch.float32 for p in parts) else parts[0].dtype
+        fused = torch.empty(sum(p.shape[0] for p in parts), self.hidden, dtype=dt, device=parts[0].device)
+        o = 0
+        for p in parts:
+            fused[o:o + p.shape[0]].copy_(p)
+            o += p.shape[0]
+        self.w_in = ops.pack_weight(fused)
+        self.w_a1 = ops.pack_weight(source.get(prefix + n["a1"]))
+        self.w_a2 = ops.pack_weight(source.get(prefix + n["a2"]))
+        self.b_a2 = source.get(prefix + n["a2_bias"]).float().contiguous()
+        self.w_norm = source.get(prefix + n["norm"]).float().contiguous()
+        self.w_o = ops.pack_weight(source.get(prefix + n["o"]))
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
+        if not cache.write:
+            raise ValueError("a recurrent mixer's state cannot be shared between layers")
+        T = x.shape[0]
+        qk, vv = self.nh * self.dk, self.nh * self.dv
+        width = 2 if ctx.act_dtype == torch.bfloat16 else 4
+        n_in = 2 * qk + (2 if self.has_gate else 1) * vv
+        with section("q|k|v|g", nbytes=width * n_in * (self.hidden + T) + width * T * self.hidden, flops=2.0 * T * self.hidden * n_in):
+            proj = ops.linear(x, self.w_in, ctx.act_dtype)
+        with section("decay logits", nbytes=width * self.rank * (self.hidden + qk) + 4 * T * qk,
+                     flops=2.0 * T * self.rank * (self.hidden + qk)):
+            z = ops.linear(ops.linear(x, self.w_a1, ctx.act_dtype), self.w_a2, torch.float32)
+        state = cache.states[0] if cache.states else cache.state
+        with section("recurrence", nbytes=lambda: 8 * ctx.n_entries * qk * self.dv + T * (width * (2 * qk + vv) + 4 * (qk + vv)),
+                     flops=4.0 * T * qk * self.dv):
+            o = ops.gla_walk(proj, 0, qk, 2 * qk, z, self.b_a2, self.tau, self.dk ** -0.5, state, ctx, self.nh, self.dk, self.dv)
+        with section("head norm + gate", nbytes=T * vv * (4 + 2 * width)):
+            y = ops.head_norm_gate(o, self.w_norm, self.eps, self.nh, self.dv, ctx.act_dtype,
+                                   proj if self.has_gate else None, 2 * qk + vv)
+        with section("o", nbytes=width * self.hidden * (vv + T) + width * T * vv, flops=2.0 * T * self.hidden * vv):
+            return ops.linear(y, self.w_o, ctx.act_dtype)

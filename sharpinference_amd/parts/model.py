@@ -2,7 +2,7 @@
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, List, Optional, Sequence
+from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
@@ -18,11 +18,15 @@ class Run:
 
     A layer may appear in several entries (its weights are used again; give each entry its own
     cache slot unless sharing is meant).  ``write=False`` makes the entry read the keys and
-    values that the slot's owner stored earlier in the same step and store nothing."""
+    values that the slot's owner stored earlier in the same step and store nothing.
+    ``add_row`` = (table, r): before the layer runs, row r of the model's tensor `table` (one of its
+    ``row_tables``, [rows, hidden]) is added to every token's residual sum, in float: a learned
+    vector that marks, say, which pass of a repeated stretch of layers begins here."""
 
     layer: int
     cache: int
     write: bool = True
+    add_row: Optional[Tuple[str, int]] = None
 
 
 class DecoderModel(Part):
@@ -37,7 +41,10 @@ class DecoderModel(Part):
                  schedule: Optional[Sequence[Run]] = None, tie_embeddings: bool = False, config=None,
                  layer_prefix: str = "model.layers.", embed_name: str = "model.embed_tokens.weight",
                  norm_prefix: str = "model.norm.", head_name: str = "lm_head.weight", embedding_scale: float = 1.0,
-                 logit_scale: float = 1.0, logit_softcap: Optional[float] = None):
+                 logit_scale: float = 1.0, logit_softcap: Optional[float] = None,
+                 row_tables: Optional[Dict[str, int]] = None):
+        self.row_tables: Dict[str, int] = dict(row_tables or {})      # name -> rows of a [rows, hidden] tensor
+        self._row_table_f32: Dict[str, torch.Tensor] = {}
         self.vocab_size, self.hidden = int(vocab_size), int(hidden)
         self.blocks = list(blocks)
         self.final_norm = final_norm
@@ -62,6 +69,10 @@ class DecoderModel(Part):
             if not 0 <= r.cache < n_slots:
                 raise ValueError(f"schedule names cache slot {r.cache} out of range")
             spec = self.blocks[r.layer].cache_spec()
+            if r.add_row is not None:
+                name, row = r.add_row
+                if name not in self.row_tables or not 0 <= row < self.row_tables[name]:
+                    raise ValueError(f"schedule adds row {row} of {name!r}, which the model does not have")
             if r.write:
                 if r.cache in owner:
                     raise ValueError(f"cache slot {r.cache} is written by two entries of the schedule")
@@ -103,6 +114,8 @@ class DecoderModel(Part):
         for i, b in enumerate(self.blocks):
             out.update(b.param_specs(f"{self.layer_prefix}{i}."))
         out.update(self.final_norm.param_specs(self.norm_prefix))
+        for name, rows in self.row_tables.items():
+            out[name] = ParamSpec((rows, self.hidden))
         if not self.tie_embeddings:
             out[self.head_name] = ParamSpec((self.vocab_size, self.hidden))
         return out
@@ -112,6 +125,7 @@ class DecoderModel(Part):
         for i, b in enumerate(self.blocks):
             b.load(f"{self.layer_prefix}{i}.", source)
         self.final_norm.load(self.norm_prefix, source)
+        self._row_table_f32 = {name: source.get(name).float().contiguous() for name in self.row_tables}
         # the head also in the order the few-rows kernel streams it (the rows stay for many-row steps
         # and, when tied, for the embedding gather)
         self.head = ops.pack_weight(self.embed if self.tie_embeddings else source.get(self.head_name))
@@ -129,8 +143,13 @@ class DecoderModel(Part):
             stream = ResidualStream(ops.embed_gather(ctx.token_ids, self.embed, scale=self.embedding_scale))
         for r in self.schedule:
             c = caches[r.cache]
+            if r.add_row is not None:
+                if stream.pending is not None:
+                    raise ValueError("a row can be added only where no branch output is pending")
+                with section("row added to the stream", nbytes=ctx.n_tokens * self.hidden * 8):
+                    ops.add_bias(stream.h, self._row_table_f32[r.add_row[0]][r.add_row[1]])
             if not r.write:
-                c = LayerCache(c.group, c.k, c.v, c.state, write=False)
+                c = LayerCache(c.group, c.k, c.v, c.state, write=False, states=c.states)
             self.blocks[r.layer].forward(stream, ctx, c)
         if logit_rows is None or logit_rows.numel() == 0:
             return None

@@ -4,10 +4,12 @@ What a mixer needs of a rotary encoding is small: ``table(device)`` (float32 fre
 rotated pair), ``pair_layout`` ("interleaved": pairs (2i, 2i+1); "half": pairs (i, i + r/2)) and
 ``rotary_dim`` (r: how many leading elements of a head rotate).  Any object with these three can
 be handed to the attention mixer; each layer may hold its own (another base, another width).
+``magnitude`` (1 unless an encoding says otherwise) multiplies cos and sin alike.
 """
 from __future__ import annotations
 
 import math
+from dataclasses import dataclass
 from typing import Optional
 
 import torch
@@ -15,6 +17,28 @@ import torch
 from .base import Part
 
 PAIR_LAYOUTS = ("interleaved", "half")
+
+
+@dataclass(frozen=True)
+class WavelengthScaling:
+    """The llama3 rule's four numbers, under the names ``Rotary`` reads them by."""
+
+    factor: float
+    low_freq_factor: float
+    high_freq_factor: float
+    original_max_position_embeddings: float
+
+
+@dataclass(frozen=True)
+class YarnScaling:
+    """YaRN: `factor` stretches the slow pairs; a pair that turns more than `fast` times within the
+    `original` context keeps its frequency, one that turns fewer than `slow` times is divided by
+    the factor, and the pairs between are blended along a ramp over the pair index."""
+
+    factor: float
+    original: float
+    fast: float
+    slow: float
 
 
 class Rotary(Part):
@@ -38,6 +62,7 @@ class Rotary(Part):
             raise ValueError(f"pair_layout {pair_layout!r} is not known ({', '.join(PAIR_LAYOUTS)})")
         self.head_dim, self.theta, self.scaling = int(head_dim), float(theta), scaling
         self.pair_layout, self.rotary_dim = pair_layout, rotary_dim
+        self.magnitude = 1.0
         self._table: Optional[torch.Tensor] = None
 
     def frequencies(self) -> torch.Tensor:
@@ -70,3 +95,38 @@ class RotaryInterleaved(Rotary):
 
     def __init__(self, head_dim: int, theta: float, scaling=None):
         super().__init__(head_dim, theta, scaling, "interleaved", None)
+
+
+YARN_MAGNITUDE_SLOPE = 0.1
+
+
+class YarnRotary(Rotary):
+    """Rotary positions with YaRN's interpolation.  With r rotated elements and base b, the pair
+    that turns n times within the original context o has the (real-valued) index
+    i(n) = r ln(o / (2 pi n)) / (2 ln b); lo = max(floor(i(fast)), 0), hi = min(ceil(i(slow)), r - 1),
+    ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), and pair i turns with
+    f_i / factor * ramp_i + f_i * (1 - ramp_i).  cos and sin are both multiplied by
+    0.1 ln(factor) + 1 (``magnitude``), which scales every score of rotated parts by its square."""
+
+    def __init__(self, head_dim: int, theta: float, scaling: YarnScaling, pair_layout: str = "interleaved",
+                 rotary_dim: Optional[int] = None):
+        super().__init__(head_dim, theta, None, pair_layout, rotary_dim)
+        if not scaling.factor > 0 or not scaling.original > 0 or not scaling.fast > 0 or not scaling.slow > 0:
+            raise ValueError("YaRN scaling: factor, original, fast and slow must be positive")
+        self.yarn = scaling
+        self.magnitude = YARN_MAGNITUDE_SLOPE * math.log(scaling.factor) + 1.0
+
+    def frequencies(self) -> torch.Tensor:
+        rd, s = self.rotary_dim, self.yarn
+
+        def pair_index(turns: float) -> float:
+            return rd * math.log(s.original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+
+        lo = max(math.floor(pair_index(s.fast)), 0)
+        hi = min(math.ceil(pair_index(s.slow)), rd - 1)
+        freqs = []
+        for i in range(rd // 2):
+            f = math.pow(self.theta, -2.0 * i / rd)
+            ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            freqs.append(f / s.factor * ramp + f * (1.0 - ramp))
+        return torch.tensor(freqs, dtype=torch.float64).to(torch.float32)
