@@ -12,7 +12,9 @@ prefill and one decode step, from event pairs.  ``--shape maverick8`` and ``--sh
 two other workloads instead (128 experts alternating with dense layers at batch 64; 32,768-token
 prompts read in 4,096-token portions beside decoding requests) and print a JSON line of their own;
 ``--shape kuvonex`` runs Kuvonex layers (latent attention, routed experts in groups) at two sizes,
-each beside Llama 4 layers of the same width, heads and experts, with the kernel-class tables of both.
+each beside Llama 4 layers of the same width, heads and experts, with the kernel-class tables of both;
+``--shape pazatar`` does the same for Pazatar layers (attention that norms before it rotates, gated linear
+attention beside it, dense feed-forwards) beside Llama 4 layers with dense feed-forwards.
 """
 from __future__ import annotations
 
@@ -493,18 +495,18 @@ def llama4_config_like(z: dict) -> dict:
     return cfg
 
 
-def run_kuvonex(args) -> int:
-    """Prefill of one 2,048-token prompt and decode at batch 8 and 64 for the Kuvonex design at two
-    sizes, each beside Llama 4 layers of the same width, heads, experts and expert width (random
-    weights), with the per-kernel-class tables of one prefill and one decode step of both."""
+def _beside(args, sizes: dict, pairs) -> tuple:
+    """Prefill of one prompt and decode at batch 8 and 64 for every size and every (model, configuration
+    maker) of `pairs`, with the per-kernel-class tables of one prefill and one decode step of each."""
     import torch
     from sharpinference_amd.engine import Engine
 
     P, steps, warm = args.prompt_len, min(args.steps, 48), 4
     per_req = (P + steps + warm + 16 + args.page_size - 1) // args.page_size * args.page_size + 2 * args.page_size
     rows = []
-    for size, z in KUVONEX_SIZES.items():
-        for model, cfg in (("kuvonex", kuvonex_config(z)), ("llama4", llama4_config_like(z))):
+    for size, z in sizes.items():
+        for model, make in pairs:
+            cfg = make(z)
             t0 = time.time()
             eng = Engine(config=cfg, weight_seed=2, dtype="bfloat16", device="cuda:0", max_model_len=CONTEXT, max_num_seqs=64,
                          max_tokens_per_step=8192, kv_tokens=64 * per_req, page_size=args.page_size,
@@ -532,12 +534,75 @@ def run_kuvonex(args) -> int:
             rows.append(row)
             del eng
             torch.cuda.empty_cache()
+    return rows, P, steps, warm
+
+
+def run_kuvonex(args) -> int:
+    """Prefill of one 2,048-token prompt and decode at batch 8 and 64 for the Kuvonex design at two
+    sizes, each beside Llama 4 layers of the same width, heads, experts and expert width (random
+    weights), with the per-kernel-class tables of one prefill and one decode step of both."""
+    rows, P, steps, warm = _beside(args, KUVONEX_SIZES, (("kuvonex", kuvonex_config), ("llama4", llama4_config_like)))
     k0 = rows[0]
     out = {"metric": "decode tok/s at batch 8 (Kuvonex, width 2048, 4 layers, 2,048-token prompts)", "value": k0["decode_b8_tok_s"],
            "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": k0["decode_b8_ms_per_step"],
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
            "config": {"model": "kuvonex-random beside llama4-random at equal sizes", "global_batch": 8, "seq_len": CONTEXT,
                       "parallelism": "single-gpu", "prompt_len": P, "sizes": KUVONEX_SIZES},
+           "rows": rows}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+# ---------------------------------------------------------------------------
+# Pazatar beside Llama 4 with dense feed-forwards at equal sizes
+# ---------------------------------------------------------------------------
+# width, layers (attention and parallel layers in turn), heads of 128 over kv heads, the gated linear mixer's heads of
+# 128 key and 128 value channels, feed-forward width, vocabulary
+PAZATAR_SIZES = {
+    "w2048": dict(width=2048, layers=4, heads=16, kv_heads=4, ff=8192, vocab=32000, chunk=1024, decay_rank=64),
+    "w4096": dict(width=4096, layers=2, heads=32, kv_heads=8, ff=14336, vocab=32000, chunk=1024, decay_rank=128),
+}
+
+
+def pazatar_config(z: dict) -> dict:
+    attention = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                 "mask": {"size": z["chunk"]},
+                 "rot": {"base": 10000.0, "dims": 128, "scaling": {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}
+    left = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "conv": 4,
+            "softcap": 50.0, "mask": {"size": z["chunk"] // 2},
+            "rot": {"base": 20000.0, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 2048}}}
+    right = {"heads": z["heads"], "dim": 128, "vdim": 128, "tau": 16.0, "decay_rank": z["decay_rank"]}
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    layers = [{"type": "attention", "mixer": attention, "mlp": mlp} if i % 2 == 0 else
+              {"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp} for i in range(z["layers"])]
+    return {"architecture": "Pazatar", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-5}, "layers": layers,
+            "loop": {"start": 0, "stop": z["layers"], "times": 1}}
+
+
+def llama4_dense_like(z: dict) -> dict:
+    """Llama 4 layers of the same width, heads and kv heads, every feed-forward dense (gated: three
+    matrices of the width where the other design has two) and every layer chunked."""
+    cfg = dict(SCOUT)
+    cfg.update({"hidden_size": z["width"], "num_hidden_layers": z["layers"], "num_attention_heads": z["heads"],
+                "num_key_value_heads": z["kv_heads"], "head_dim": 128, "vocab_size": z["vocab"],
+                "intermediate_size": z["ff"], "intermediate_size_mlp": z["ff"], "num_local_experts": 1,
+                "num_experts_per_tok": 1, "interleave_moe_layer_step": z["layers"] + 1, "rope_scaling": None,
+                "attention_chunk_size": z["chunk"], "no_rope_layers": [1] * z["layers"], "max_position_embeddings": CONTEXT})
+    return cfg
+
+
+def run_pazatar(args) -> int:
+    """Prefill of one 2,048-token prompt and decode at batch 8 and 64 for the Pazatar design at two
+    sizes (attention layers and parallel layers in turn, random weights), each beside Llama 4
+    layers of the same width and heads with dense feed-forwards, with the per-kernel-class tables
+    of one prefill and one decode step of both."""
+    rows, P, steps, warm = _beside(args, PAZATAR_SIZES, (("pazatar", pazatar_config), ("llama4", llama4_dense_like)))
+    k0 = rows[0]
+    out = {"metric": "decode tok/s at batch 8 (Pazatar, width 2048, 4 layers, 2,048-token prompts)", "value": k0["decode_b8_tok_s"],
+           "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": k0["decode_b8_ms_per_step"],
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+           "config": {"model": "pazatar-random beside llama4-random (dense feed-forwards) at equal sizes", "global_batch": 8,
+                      "seq_len": CONTEXT, "parallelism": "single-gpu", "prompt_len": P, "sizes": PAZATAR_SIZES},
            "rows": rows}
     print(json.dumps(out), flush=True)
     return 0
@@ -556,8 +621,8 @@ def main() -> int:
     ap.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel instead of replaying a HIP graph")
     ap.add_argument("--no-peaks", action="store_true", help="skip the two measuring kernels (pure read, matrix-core loop)")
     ap.add_argument("--profile", action="store_true", help="also print ms / bytes / GB/s per kernel class of one prefill and one decode step")
-    ap.add_argument("--shape", default="scout", choices=["scout", "maverick8", "long16", "kuvonex"],
-                    help="scout: the headline run; maverick8 / long16: two other workloads; kuvonex: the Kuvonex design beside "
+    ap.add_argument("--shape", default="scout", choices=["scout", "maverick8", "long16", "kuvonex", "pazatar"],
+                    help="scout: the headline run; maverick8 / long16: two other workloads; kuvonex / pazatar: that design beside "
                          "Llama 4 layers of equal size; each prints a JSON line of its own")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -569,6 +634,8 @@ def main() -> int:
         return run_long16(args)
     if args.shape == "kuvonex":
         return run_kuvonex(args)
+    if args.shape == "pazatar":
+        return run_pazatar(args)
 
     import torch  # noqa: F401
 

@@ -3,84 +3,198 @@
 // walked token by token in float.  The state of a request lives in its state slot
 // [slots, heads, dk, dv] (float) and is carried from step to step.
 //
-// A wave owns kCols value columns of one head of one entry: the columns of S are independent of
-// each other, so an entry's work is spread over heads x ceil(dv / kCols) waves, and the walk along
-// the entry's tokens is the only thing that is sequential.  Lane (g, j) holds rows g, g + 4,
-// g + 8, ... of column j (RPL rows a lane).  Per token the lane scales its rows by alpha, adds
-// k[row] * v[j], and sums S[row][j] * q[row] over its rows; the four row groups are then added by
-// two exchanges between lanes.  Every sum's order depends on (dk, dv) alone: a token's output has
-// the same bits however its request's tokens were cut into steps.
+// A block owns kCols value columns of one head of one entry: the columns of S are independent of
+// each other, so an entry's work is spread over heads x ceil(dv / kCols) blocks, and the walk along
+// the entry's tokens is the only thing that is sequential.  The block is two waves.  One walks:
+// lane (g, j) holds RPL consecutive rows of column j (rows g * RPL ...); per token it scales its rows
+// by alpha, adds k[row] * v[j], and sums S[row][j] * q[row] over its rows; the row groups are then
+// added by exchanges between lanes.  The other wave runs a stage ahead: it fetches q, k, v and the
+// decays of the next kStage tokens (16 bytes a load where sizes and offsets are multiples of
+// eight) and leaves them in the other half of LDS, so that the walking wave reads LDS only and
+// never waits for memory.  Every sum's order depends on (dk, dv) alone: a token's output has the
+// same bits however its request's tokens were cut into steps.
 //
-// q, k, alpha of kStage tokens are staged in LDS by the whole wave (alpha computed there, in
-// float, as exp(log_sigmoid(z + bias) / tau)), so the walk itself reads LDS broadcasts only.
+// The decays are made from their logits once per (token, channel) by a kernel of their own, in
+// float: alpha = exp(log_sigmoid(z + bias) / tau), in place over the logits.
 #include "common.h"
 
-constexpr int kCols = 16;      // value columns a wave owns
-constexpr int kGroups = 4;     // row groups (kWave / kCols)
-constexpr int kStage = 8;      // tokens staged at a time
+constexpr int kCols = 8;                 // value columns a block owns
+constexpr int kGroups = kWave / kCols;   // row groups
 
 // log(sigmoid(z)) without overflow: min(z, 0) - log1p(exp(-|z|))
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
-template <typename T, int RPL>
-__global__ __launch_bounds__(kWave) void gla_walk_kernel(
-    const T* __restrict__ proj, int stride, int q_off, int k_off, int v_off, const float* __restrict__ z,
-    const float* __restrict__ z_bias, float inv_tau, float q_scale, float* __restrict__ state,
+__global__ void gla_decays_kernel(float* __restrict__ z, const float* __restrict__ bias, float inv_tau, size_t n, int N) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    z[i] = expf(log_sigmoid(z[i] + bias[i % N]) * inv_tau);
+}
+
+// The decays straight from the narrow middle of their projection: alpha[t, c] = sigmoid(sum_r a1[t, r]
+// W[c, r] + bias[c])^(1 / tau).  a1 are `rank` columns of a wider row (the step's fused projection).  A
+// block takes kDecayTokens tokens and 256 channels; a thread one channel, whose weight row it reads
+// once for all the block's tokens; the sum is one ascending chain of float FMAs.
+constexpr int kDecayTokens = 8;
+constexpr int kDecayMaxRank = 256;
+
+template <typename T>
+__global__ __launch_bounds__(256) void gla_decays_fused_kernel(const T* __restrict__ proj, int stride, int a_off, int rank,
+                                                               const T* __restrict__ w, const float* __restrict__ bias,
+                                                               float inv_tau, float* __restrict__ alpha, int n_tokens, int N) {
+  __shared__ float a1[kDecayTokens][kDecayMaxRank];
+  const int t0 = blockIdx.x * kDecayTokens;
+  const int nt = min(kDecayTokens, n_tokens - t0);
+  for (int i = threadIdx.x; i < kDecayTokens * rank; i += blockDim.x) {
+    const int tt = i / rank, r = i % rank;
+    a1[tt][r] = tt < nt ? to_f32<T>(proj[(size_t)(t0 + tt) * stride + a_off + r]) : 0.f;
+  }
+  __syncthreads();
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= N) return;
+  float acc[kDecayTokens];
+#pragma unroll
+  for (int tt = 0; tt < kDecayTokens; ++tt) acc[tt] = 0.f;
+  const T* wr = w + (size_t)c * rank;
+  for (int r = 0; r < rank; ++r) {
+    const float wv = to_f32<T>(wr[r]);
+#pragma unroll
+    for (int tt = 0; tt < kDecayTokens; ++tt) acc[tt] = fmaf(a1[tt][r], wv, acc[tt]);
+  }
+  const float b = bias[c];
+#pragma unroll
+  for (int tt = 0; tt < kDecayTokens; ++tt)
+    if (tt < nt) alpha[(size_t)(t0 + tt) * N + c] = expf(log_sigmoid(acc[tt] + b) * inv_tau);
+}
+
+template <typename T, int RPL, bool VEC>
+__global__ __launch_bounds__(2 * kWave) void gla_walk_kernel(
+    const T* __restrict__ proj, int stride, int q_off, int k_off, int v_off, const float* __restrict__ alpha,
+    float q_scale, float* __restrict__ state,
     const int* __restrict__ state_slots, const int* __restrict__ cu_tokens, float* __restrict__ out, int nh, int dk,
     int dv) {
-  __shared__ float qs[kStage][RPL * kGroups];
-  __shared__ float ks[kStage][RPL * kGroups];
-  __shared__ float as[kStage][RPL * kGroups];
+  constexpr int DKP = RPL * kGroups;               // rows the lanes cover; rows beyond dk stay zero
+  constexpr int kStage = DKP <= 128 ? 16 : 8;      // tokens staged at a time (two stages fit in LDS)
+  __shared__ __attribute__((aligned(16))) float qs[2][kStage][DKP];
+  __shared__ __attribute__((aligned(16))) float ks[2][kStage][DKP];
+  __shared__ __attribute__((aligned(16))) float as[2][kStage][DKP];
+  __shared__ float vs[2][kStage][kCols];
   const int e = blockIdx.z, h = blockIdx.y, c0 = blockIdx.x * kCols;
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & (kWave - 1);
+  const bool walker = threadIdx.x < kWave;
   const int j = lane % kCols, g = lane / kCols;
   const int col = c0 + j;
   const bool col_ok = col < dv;
   const int first = cu_tokens[e], len = cu_tokens[e + 1] - first;
   float* S = state + (((size_t)state_slots[e] * nh + h) * dk) * dv;
   float s[RPL];
+  if (walker) {
 #pragma unroll
-  for (int r = 0; r < RPL; ++r) {
-    const int rowi = g + kGroups * r;
-    s[r] = (col_ok && rowi < dk) ? S[(size_t)rowi * dv + col] : 0.f;
+    for (int r = 0; r < RPL; ++r) {
+      const int rowi = g * RPL + r;
+      s[r] = (col_ok && rowi < dk) ? S[(size_t)rowi * dv + col] : 0.f;
+    }
   }
-  constexpr int DKP = RPL * kGroups;   // rows the lanes cover; rows beyond dk stay zero
-  for (int t0 = 0; t0 < len; t0 += kStage) {
+  auto stage = [&](int t0, int buf) {
     const int nt = min(kStage, len - t0);
-    __syncthreads();
-    for (int i = lane; i < nt * DKP; i += kWave) {
-      const int tt = i / DKP, d = i % DKP;
-      const size_t tok = (size_t)(first + t0 + tt);
-      float qv = 0.f, kv = 0.f, av = 1.f;
-      if (d < dk) {
-        qv = to_f32<T>(proj[tok * stride + q_off + h * dk + d]) * q_scale;
-        kv = to_f32<T>(proj[tok * stride + k_off + h * dk + d]);
-        av = expf(log_sigmoid(z[tok * (size_t)(nh * dk) + h * dk + d] + z_bias[h * dk + d]) * inv_tau);
-      }
-      qs[tt][d] = qv;
-      ks[tt][d] = kv;
-      as[tt][d] = av;
-    }
-    __syncthreads();
-    for (int tt = 0; tt < nt; ++tt) {
-      const size_t tok = (size_t)(first + t0 + tt);
-      const float v = col_ok ? to_f32<T>(proj[tok * stride + v_off + h * dv + col]) : 0.f;
-      float o = 0.f;
+    if constexpr (VEC) {     // dk, the row strides and the offsets are multiples of eight
+      // every load of the stage is requested before the first is used, none behind a branch (addresses
+      // are clamped into the stage and what lies outside is replaced afterwards)
+      constexpr int ITER = (kStage * (DKP / 8) + kWave - 1) / kWave;
+      float qv[ITER][8], kv[ITER][8], av[ITER][8];
 #pragma unroll
-      for (int r = 0; r < RPL; ++r) {
-        const int rowi = g + kGroups * r;
-        s[r] = fmaf(as[tt][rowi], s[r], ks[tt][rowi] * v);
-        o = fmaf(s[r], qs[tt][rowi], o);
+      for (int it = 0; it < ITER; ++it) {
+        const int i = lane + it * kWave;
+        const int tt = min(i / (DKP / 8), nt - 1), d = min((i % (DKP / 8)) * 8, dk - 8);
+        const size_t tok = (size_t)(first + t0 + tt);
+        load8(proj + tok * stride + q_off + h * dk + d, qv[it]);
+        load8(proj + tok * stride + k_off + h * dk + d, kv[it]);
+        load8(alpha + tok * (size_t)(nh * dk) + h * dk + d, av[it]);
       }
-      o += __shfl_xor(o, 16, kWave);
-      o += __shfl_xor(o, 32, kWave);
-      if (g == 0 && col_ok) out[tok * (size_t)(nh * dv) + h * dv + col] = o;
+#pragma unroll
+      for (int it = 0; it < ITER; ++it) {
+        const int i = lane + it * kWave;
+        const int tt = i / (DKP / 8), d = (i % (DKP / 8)) * 8;
+        if (tt >= kStage) continue;
+        const bool in = d < dk;
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+          qv[it][x] = in ? qv[it][x] * q_scale : 0.f;
+          kv[it][x] = in ? kv[it][x] : 0.f;
+          av[it][x] = in ? av[it][x] : 1.f;
+        }
+        store8(&qs[buf][tt][d], qv[it]);
+        store8(&ks[buf][tt][d], kv[it]);
+        store8(&as[buf][tt][d], av[it]);
+      }
+    } else {
+      for (int i = lane; i < nt * DKP; i += kWave) {
+        const int tt = i / DKP, d = i % DKP;
+        const size_t tok = (size_t)(first + t0 + tt);
+        float qv = 0.f, kv = 0.f, av = 1.f;
+        if (d < dk) {
+          qv = to_f32<T>(proj[tok * stride + q_off + h * dk + d]) * q_scale;
+          kv = to_f32<T>(proj[tok * stride + k_off + h * dk + d]);
+          av = alpha[tok * (size_t)(nh * dk) + h * dk + d];
+        }
+        qs[buf][tt][d] = qv;
+        ks[buf][tt][d] = kv;
+        as[buf][tt][d] = av;
+      }
     }
+    for (int i = lane; i < nt * kCols; i += kWave) {
+      const int tt = i / kCols, c = c0 + i % kCols;
+      vs[buf][tt][i % kCols] = c < dv ? to_f32<T>(proj[(size_t)(first + t0 + tt) * stride + v_off + h * dv + c]) : 0.f;
+    }
+  };
+  if (!walker) stage(0, 0);
+  __syncthreads();
+  int buf = 0;
+  for (int t0 = 0; t0 < len; t0 += kStage, buf ^= 1) {
+    if (!walker) {
+      if (t0 + kStage < len) stage(t0 + kStage, buf ^ 1);
+    } else {
+      const int nt = min(kStage, len - t0);
+      auto one_token = [&](int tt) {
+        const float v = vs[buf][tt][j];
+        const float* qrow = &qs[buf][tt][g * RPL];
+        const float* krow = &ks[buf][tt][g * RPL];
+        const float* arow = &as[buf][tt][g * RPL];
+        float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+        for (int r = 0; r < RPL; r += 4) {
+          const float4 a4 = *reinterpret_cast<const float4*>(arow + r);
+          const float4 k4 = *reinterpret_cast<const float4*>(krow + r);
+          const float4 q4 = *reinterpret_cast<const float4*>(qrow + r);
+          s[r + 0] = fmaf(a4.x, s[r + 0], k4.x * v);
+          o0 = fmaf(s[r + 0], q4.x, o0);
+          s[r + 1] = fmaf(a4.y, s[r + 1], k4.y * v);
+          o1 = fmaf(s[r + 1], q4.y, o1);
+          s[r + 2] = fmaf(a4.z, s[r + 2], k4.z * v);
+          o0 = fmaf(s[r + 2], q4.z, o0);
+          s[r + 3] = fmaf(a4.w, s[r + 3], k4.w * v);
+          o1 = fmaf(s[r + 3], q4.w, o1);
+        }
+        float o = o0 + o1;
+        o += __shfl_xor(o, 8, kWave);
+        o += __shfl_xor(o, 16, kWave);
+        o += __shfl_xor(o, 32, kWave);
+        if (g == 0 && col_ok) out[(size_t)(first + t0 + tt) * (size_t)(nh * dv) + h * dv + col] = o;
+      };
+      if (nt == kStage) {
+        // a full stage, unrolled: the LDS reads of the tokens ahead are requested while this one is summed
+#pragma unroll
+        for (int tt = 0; tt < kStage; ++tt) one_token(tt);
+      } else {
+        for (int tt = 0; tt < nt; ++tt) one_token(tt);
+      }
+    }
+    __syncthreads();
   }
+  if (walker) {
 #pragma unroll
-  for (int r = 0; r < RPL; ++r) {
-    const int rowi = g + kGroups * r;
-    if (col_ok && rowi < dk) S[(size_t)rowi * dv + col] = s[r];
+    for (int r = 0; r < RPL; ++r) {
+      const int rowi = g * RPL + r;
+      if (col_ok && rowi < dk) S[(size_t)rowi * dv + col] = s[r];
+    }
   }
 }
 
@@ -112,39 +226,79 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
 }
 
 template <typename T>
-static int launch_walk(const void* proj, int stride, int q_off, int k_off, int v_off, const float* z, const float* z_bias,
-                       float inv_tau, float q_scale, float* state, const int* state_slots, const int* cu_tokens,
-                       float* out, int n_entries, int nh, int dk, int dv, hipStream_t stream) {
+static int launch_walk(const void* proj, int stride, int q_off, int k_off, int v_off, const float* alpha, float q_scale,
+                       float* state, const int* state_slots, const int* cu_tokens, float* out, int n_entries, int nh,
+                       int dk, int dv, hipStream_t stream) {
   dim3 grid(ceil_div(dv, kCols), nh, n_entries);
-#define WALK(RPL)                                                                                                   \
-  gla_walk_kernel<T, RPL><<<grid, kWave, 0, stream>>>((const T*)proj, stride, q_off, k_off, v_off, z, z_bias, inv_tau, \
-                                                      q_scale, state, state_slots, cu_tokens, out, nh, dk, dv)
-  if (dk <= 32) WALK(8);
-  else if (dk <= 64) WALK(16);
-  else if (dk <= 128) WALK(32);
-  else if (dk <= 256) WALK(64);
+  const bool vec = dk % 8 == 0 && stride % 8 == 0 && q_off % 8 == 0 && k_off % 8 == 0 &&
+                   ((uintptr_t)proj % 32 == 0) && ((uintptr_t)alpha % 32 == 0);
+#define WALK(RPL)                                                                                                    \
+  do {                                                                                                               \
+    if (vec)                                                                                                         \
+      gla_walk_kernel<T, RPL, true><<<grid, 2 * kWave, 0, stream>>>((const T*)proj, stride, q_off, k_off, v_off, alpha, \
+                                                                    q_scale, state, state_slots, cu_tokens, out, nh, dk, dv); \
+    else                                                                                                             \
+      gla_walk_kernel<T, RPL, false><<<grid, 2 * kWave, 0, stream>>>((const T*)proj, stride, q_off, k_off, v_off, alpha, \
+                                                                     q_scale, state, state_slots, cu_tokens, out, nh, dk, dv); \
+  } while (0)
+  if (dk <= 32) WALK(4);
+  else if (dk <= 64) WALK(8);
+  else if (dk <= 128) WALK(16);
+  else if (dk <= 256) WALK(32);
   else return SHARPI_ERR_ARG;
 #undef WALK
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }
 
+// z float [n_rows, N]: decay logits, turned in place into decays sigmoid(z + bias)^(1 / tau), bias [N].
+SHARPI_EXPORT int sharpi_gla_decays(float* z, const float* bias, float tau, int n_rows, int N, hipStream_t stream) {
+  if (n_rows <= 0) return SHARPI_OK;
+  if (N <= 0 || !(tau > 0.f) || !bias) return SHARPI_ERR_ARG;
+  const size_t n = (size_t)n_rows * N;
+  gla_decays_kernel<<<(unsigned)min((size_t)8192, (n + 255) / 256), 256, 0, stream>>>(z, bias, 1.0f / tau, n, N);
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
+// proj [T, stride] of `dtype`: its columns a_off .. a_off + rank are the narrow middle of the decay
+// projection; w [N, rank] of the same dtype, bias float [N]; alpha float [T, N] receives
+// sigmoid(a1 w^T + bias)^(1 / tau).
+SHARPI_EXPORT int sharpi_gla_decays_fused(const void* proj, int dtype, int stride, int a_off, int rank, const void* w,
+                                          const float* bias, float tau, float* alpha, int n_tokens, int N,
+                                          hipStream_t stream) {
+  if (n_tokens <= 0) return SHARPI_OK;
+  if (N <= 0 || rank <= 0 || rank > kDecayMaxRank || !(tau > 0.f) || !bias || !w) return SHARPI_ERR_ARG;
+  dim3 grid(ceil_div(n_tokens, kDecayTokens), ceil_div(N, 256));
+  if (grid.y > 65535) return SHARPI_ERR_ARG;
+  if (dtype == DT_F32)
+    gla_decays_fused_kernel<float><<<grid, 256, 0, stream>>>((const float*)proj, stride, a_off, rank, (const float*)w, bias,
+                                                             1.0f / tau, alpha, n_tokens, N);
+  else if (dtype == DT_BF16)
+    gla_decays_fused_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)proj, stride, a_off, rank, (const bf16_t*)w,
+                                                              bias, 1.0f / tau, alpha, n_tokens, N);
+  else
+    return SHARPI_ERR_ARG;
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
 // proj [T, stride] of `dtype` holds q (nh * dk columns at q_off), k (at k_off) and v (nh * dv at
-// v_off); z float [T, nh * dk] are the decay logits before their bias z_bias [nh * dk]; state float
-// [slots, nh, dk, dv]; out float [T, nh * dv].  Entries (cu_tokens [entries + 1]) are walked in
-// parallel, each from the state of its slot, which is left advanced.
-SHARPI_EXPORT int sharpi_gla_walk(const void* proj, int dtype, int stride, int q_off, int k_off, int v_off, const float* z,
-                                  const float* z_bias, float tau, float q_scale, float* state, const int* state_slots,
+// v_off); alpha float [T, nh * dk] are the decays; state float [slots, nh, dk, dv]; out float
+// [T, nh * dv].  Entries (cu_tokens [entries + 1]) are walked in parallel, each from the state of
+// its slot, which is left advanced.
+SHARPI_EXPORT int sharpi_gla_walk(const void* proj, int dtype, int stride, int q_off, int k_off, int v_off,
+                                  const float* alpha, float q_scale, float* state, const int* state_slots,
                                   const int* cu_tokens, float* out, int n_entries, int nh, int dk, int dv,
                                   hipStream_t stream) {
   if (n_entries <= 0) return SHARPI_OK;
-  if (nh <= 0 || nh > 65535 || n_entries > 65535 || dk <= 0 || dk > 256 || dv <= 0 || !(tau > 0.f)) return SHARPI_ERR_ARG;
+  if (nh <= 0 || nh > 65535 || n_entries > 65535 || dk <= 0 || dk > 256 || dv <= 0) return SHARPI_ERR_ARG;
   if (dtype == DT_F32)
-    return launch_walk<float>(proj, stride, q_off, k_off, v_off, z, z_bias, 1.0f / tau, q_scale, state, state_slots,
-                              cu_tokens, out, n_entries, nh, dk, dv, stream);
+    return launch_walk<float>(proj, stride, q_off, k_off, v_off, alpha, q_scale, state, state_slots, cu_tokens, out,
+                              n_entries, nh, dk, dv, stream);
   if (dtype == DT_BF16)
-    return launch_walk<bf16_t>(proj, stride, q_off, k_off, v_off, z, z_bias, 1.0f / tau, q_scale, state, state_slots,
-                               cu_tokens, out, n_entries, nh, dk, dv, stream);
+    return launch_walk<bf16_t>(proj, stride, q_off, k_off, v_off, alpha, q_scale, state, state_slots, cu_tokens, out,
+                               n_entries, nh, dk, dv, stream);
   return SHARPI_ERR_ARG;
 }
 

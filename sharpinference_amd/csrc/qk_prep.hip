@@ -6,14 +6,18 @@
 // magnitude), and the write of keys and values into the paged cache.  Values may be the keys as
 // they were before norm and rotation (a layer without a value projection).
 //
-// One block per token.  The token's row is gathered into LDS as floats (the convolution reads up
-// to taps - 1 earlier rows: of this step where the entry has them, otherwise the tail that the
-// request's state slot carries), the sums of squares are taken in an order that depends on the
-// row alone, and everything after the projection is float arithmetic rounded once, on the way out.
+// One block per token, or, in steps of few tokens, one per (token, kv head): the block then takes
+// that kv head's key and value and the query heads that read it, so that a decode step still fills
+// the chip (what a row's sums are made of and their order do not depend on the split).  The token's
+// row is gathered into LDS as floats (the convolution reads up to taps - 1 earlier rows: of this
+// step where the entry has them, otherwise the tail that the request's state slot carries), the
+// sums of squares are taken in an order that depends on the row alone, and everything after the
+// projection is float arithmetic rounded once, on the way out.
 #include "common.h"
 
 constexpr int kPrepThreads = 256;
 constexpr int kPrepMaxTaps = 8;
+constexpr int kPrepSplitTokens = 64;  // up to so many tokens a step, a token's heads are spread over nkv blocks
 constexpr int kPrepMaxHeads = 1024;   // q heads + kv heads whose inverse norms are kept in LDS
 
 enum : int { NORM_NONE = 0, NORM_PER_HEAD = 1, NORM_WHOLE = 2 };
@@ -41,6 +45,7 @@ struct PrepArgs {
   void* v_cache;           // [pages, nkv, vd, page_size]
   const int* slot_mapping; // [T], -1: store nothing
   int page_size;
+  int parts;               // blocks a token: 1, or nkv (a kv head and its query heads each)
 };
 
 template <typename T>
@@ -49,11 +54,23 @@ __global__ __launch_bounds__(kPrepThreads) void qk_prep_kernel(PrepArgs a) {
   __shared__ float red[16];
   __shared__ float inv[kPrepMaxHeads];
   const int t = blockIdx.x;
+  // the heads this block takes: all, or kv head blockIdx.y with its query heads
+  const int per_kv = a.nh / a.nkv;
+  const int qh0 = a.parts > 1 ? blockIdx.y * per_kv : 0, qh1 = a.parts > 1 ? qh0 + per_kv : a.nh;
+  const int kh0 = a.parts > 1 ? blockIdx.y : 0, kh1 = a.parts > 1 ? kh0 + 1 : a.nkv;
+  const bool every_qk = a.norm_mode == NORM_WHOLE;   // a norm over the whole projection reads all of q and of k
   const int qn = a.nh * a.hd, kn = a.nkv * a.hd;
   const bool own_v = a.v_off >= 0;
   const int vn = own_v ? a.nkv * a.vd : 0;
   const int C = qn + kn + vn;
   const T* proj = (const T*)a.proj;
+  const bool all = a.parts == 1;                     // (then no channel or head needs asking)
+  auto mine = [&](int c) {
+    if (all) return true;
+    if (c < qn) return every_qk || (c / a.hd >= qh0 && c / a.hd < qh1);
+    if (c < qn + kn) return every_qk || ((c - qn) / a.hd >= kh0 && (c - qn) / a.hd < kh1);
+    return (c - qn - kn) / a.vd >= kh0 && (c - qn - kn) / a.vd < kh1;
+  };
 
   // 1. gather, through the convolution where there is one
   if (a.taps > 0) {
@@ -61,6 +78,7 @@ __global__ __launch_bounds__(kPrepThreads) void qk_prep_kernel(PrepArgs a) {
     const int li = t - a.cu_tokens[e];                 // the token's place in its entry
     const float* tail = a.tail + (size_t)a.state_slots[e] * (a.taps - 1) * C;
     for (int c = threadIdx.x; c < C; c += kPrepThreads) {
+      if (!mine(c)) continue;
       const int col = c < qn ? a.q_off + c : c < qn + kn ? a.k_off + (c - qn) : a.v_off + (c - qn - kn);
       float y = 0.f;
       for (int j = 0; j < a.taps; ++j) {
@@ -74,6 +92,7 @@ __global__ __launch_bounds__(kPrepThreads) void qk_prep_kernel(PrepArgs a) {
     }
   } else {
     for (int c = threadIdx.x; c < C; c += kPrepThreads) {
+      if (!mine(c)) continue;
       const int col = c < qn ? a.q_off + c : c < qn + kn ? a.k_off + (c - qn) : a.v_off + (c - qn - kn);
       row[c] = to_f32<T>(proj[(size_t)t * a.stride + col]);
     }
@@ -86,7 +105,7 @@ __global__ __launch_bounds__(kPrepThreads) void qk_prep_kernel(PrepArgs a) {
     const int page = slot / a.page_size, off = slot % a.page_size;
     T* vc = (T*)a.v_cache;
     const float* vsrc = own_v ? row + qn + kn : row + qn;
-    for (int i = threadIdx.x; i < a.nkv * a.vd; i += kPrepThreads) {
+    for (int i = kh0 * a.vd + threadIdx.x; i < kh1 * a.vd; i += kPrepThreads) {
       const int g = i / a.vd, d = i % a.vd;
       vc[(((size_t)page * a.nkv + g) * a.vd + d) * a.page_size + off] = from_f32<T>(vsrc[i]);
     }
@@ -97,6 +116,7 @@ __global__ __launch_bounds__(kPrepThreads) void qk_prep_kernel(PrepArgs a) {
   const int heads = a.nh + a.nkv;
   if (a.norm_mode == NORM_PER_HEAD) {
     for (int h = wid; h < heads; h += kPrepThreads / kWave) {
+      if (!all && !(h < a.nh ? (h >= qh0 && h < qh1) : (h - a.nh >= kh0 && h - a.nh < kh1))) continue;
       const float* x = row + (size_t)h * a.hd;         // (q heads then k heads lie back to back)
       float ss = 0.f;
       for (int d = lane; d < a.hd; d += kWave) ss = fmaf(x[d], x[d], ss);
@@ -121,6 +141,7 @@ __global__ __launch_bounds__(kPrepThreads) void qk_prep_kernel(PrepArgs a) {
   T* kc = (T*)a.k_cache;
   for (int i = threadIdx.x; i < heads * half_hd; i += kPrepThreads) {
     const int h = i / half_hd, pi = i % half_hd;
+    if (!all && !(h < a.nh ? (h >= qh0 && h < qh1) : (h - a.nh >= kh0 && h - a.nh < kh1))) continue;
     int d0, d1;
     bool turns;
     if (pi < half_r) {
@@ -204,11 +225,13 @@ SHARPI_EXPORT int sharpi_qk_prep(const void* proj, int dtype, int stride, int q_
   const int qn = nh * hd, kn = nkv * hd, vn = v_off >= 0 ? nkv * vd : 0;
   const size_t lds = (size_t)(qn + kn + vn) * sizeof(float);
   if (lds > 60 * 1024) return SHARPI_ERR_ARG;
+  const int parts = (n_tokens <= kPrepSplitTokens && nkv > 1 && nkv <= 65535 && nh % nkv == 0) ? nkv : 1;
   PrepArgs a{proj, stride, q_off, k_off, v_off, nh, nkv, hd, vd, conv_w, taps, tail, state_slots, entry_of_token,
              cu_tokens, positions, norm_mode, q_norm_w, k_norm_w, eps, rotary_dim > 0 ? inv_freq : nullptr, rotary_dim,
-             half_split, magnitude, q_out, k_cache, v_cache, slot_mapping, page_size};
-  if (dtype == DT_F32) qk_prep_kernel<float><<<n_tokens, kPrepThreads, lds, stream>>>(a);
-  else if (dtype == DT_BF16) qk_prep_kernel<bf16_t><<<n_tokens, kPrepThreads, lds, stream>>>(a);
+             half_split, magnitude, q_out, k_cache, v_cache, slot_mapping, page_size, parts};
+  dim3 pgrid(n_tokens, parts);
+  if (dtype == DT_F32) qk_prep_kernel<float><<<pgrid, kPrepThreads, lds, stream>>>(a);
+  else if (dtype == DT_BF16) qk_prep_kernel<bf16_t><<<pgrid, kPrepThreads, lds, stream>>>(a);
   else return SHARPI_ERR_ARG;
   SHARPI_CHECK_LAUNCH();
   if (taps > 0 && update_tail) {

@@ -1186,27 +1186,55 @@ def qk_prep(proj: torch.Tensor, q_off: int, k_off: int, v_off: Optional[int], nh
 GLA_MAX_KEY_DIM = 256      # key channels of a head that the walk holds (csrc/linear_attention.hip)
 
 
-def gla_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, z: torch.Tensor, z_bias: torch.Tensor, tau: float,
-             q_scale: float, state: torch.Tensor, ctx, nh: int, dk: int, dv: int) -> torch.Tensor:
+def gla_decays(z: torch.Tensor, bias: torch.Tensor, tau: float) -> torch.Tensor:
+    """Decay logits z float32 [T, N] turned IN PLACE into decays sigmoid(z + bias)^(1 / tau) (bias
+    float32 [N]): log_sigmoid, the division by tau and the exponential in float."""
+    _dev(z, bias)
+    _need(z.dtype == torch.float32 and z.dim() == 2 and bias.dtype == torch.float32 and bias.shape == (z.shape[1],) and tau > 0,
+          "gla_decays: z float32 [T, N], bias float32 [N], tau positive")
+    _run("sharpi_gla_decays", _ptr(z), _ptr(bias), float(tau), z.shape[0], z.shape[1], _stream())
+    return z
+
+
+GLA_FUSED_DECAY_MAX_RANK = 256   # csrc/linear_attention.hip kDecayMaxRank
+
+
+def gla_decays_from_middle(proj: torch.Tensor, a_off: int, rank: int, w: torch.Tensor, bias: torch.Tensor, tau: float) -> torch.Tensor:
+    """Decays sigmoid(a1 w^T + bias)^(1 / tau), float32 [T, N], straight from the narrow middle a1 of
+    their projection: columns a_off .. a_off + rank of proj [T, M]; w [N, rank] of proj's dtype, bias
+    float32 [N].  One kernel: the product as ascending float chains, then log_sigmoid, the division
+    by tau and the exponential in float."""
+    _dev(proj, w, bias)
+    T, M = proj.shape
+    N = w.shape[0]
+    _need(w.dtype == proj.dtype and w.shape == (N, rank) and 0 <= a_off and a_off + rank <= M and 1 <= rank <= GLA_FUSED_DECAY_MAX_RANK,
+          f"gla_decays_from_middle: w [N, rank] of proj's dtype, rank 1..{GLA_FUSED_DECAY_MAX_RANK}, its columns inside proj")
+    _need(bias.dtype == torch.float32 and bias.shape == (N,) and tau > 0, "gla_decays_from_middle: bias float32 [N], tau positive")
+    alpha = torch.empty(T, N, dtype=torch.float32, device=proj.device)
+    _run("sharpi_gla_decays_fused", _ptr(proj), _code(proj.dtype), M, int(a_off), int(rank), _ptr(w), _ptr(bias), float(tau),
+         _ptr(alpha), T, N, _stream())
+    return alpha
+
+
+def gla_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, alpha: torch.Tensor, q_scale: float,
+             state: torch.Tensor, ctx, nh: int, dk: int, dv: int) -> torch.Tensor:
     """The recurrence S_t = diag(alpha_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per head, token by
     token along every entry of the step, from and into state [slots, nh, dk, dv] (float32) at the
     entries' state slots.  q, k (nh*dk columns each) and v (nh*dv) are columns of proj [T, N]; q is
-    multiplied by q_scale; alpha = sigmoid(z + z_bias)^(1/tau) with z float32 [T, nh*dk].  Returns
-    o float32 [T, nh*dv]."""
-    _dev(proj, z, z_bias, state)
+    multiplied by q_scale; alpha float32 [T, nh*dk] are the decays.  Returns o float32 [T, nh*dv]."""
+    _dev(proj, alpha, state)
     T, N = proj.shape
     _need(1 <= dk <= GLA_MAX_KEY_DIM and dv >= 1 and nh >= 1, f"gla_walk: key channels 1..{GLA_MAX_KEY_DIM}")
     _need(min(q_off, k_off, v_off) >= 0 and max(q_off, k_off) + nh * dk <= N and v_off + nh * dv <= N,
           "gla_walk: q, k and v columns must lie inside proj")
-    _need(z.dtype == torch.float32 and z.shape == (T, nh * dk) and z_bias.dtype == torch.float32 and z_bias.shape == (nh * dk,),
-          "gla_walk: z float32 [T, nh*dk] and z_bias float32 [nh*dk] wanted")
+    _need(alpha.dtype == torch.float32 and alpha.shape == (T, nh * dk), "gla_walk: alpha float32 [T, nh*dk] wanted")
     _need(state.dtype == torch.float32 and state.dim() == 4 and tuple(state.shape[1:]) == (nh, dk, dv),
           "gla_walk: state must be float32 [slots, nh, dk, dv]")
     _need(ctx.state_slots.shape == (ctx.n_entries,) and ctx.cu_tokens.shape == (ctx.n_entries + 1,) and ctx.n_tokens == T,
           "gla_walk: the step's per-entry arrays do not fit")
     out = torch.empty(T, nh * dv, dtype=torch.float32, device=proj.device)
-    _run("sharpi_gla_walk", _ptr(proj), _code(proj.dtype), N, int(q_off), int(k_off), int(v_off), _ptr(z), _ptr(z_bias),
-         float(tau), float(q_scale), _ptr(state), _ptr(ctx.state_slots), _ptr(ctx.cu_tokens), _ptr(out), ctx.n_entries,
+    _run("sharpi_gla_walk", _ptr(proj), _code(proj.dtype), N, int(q_off), int(k_off), int(v_off), _ptr(alpha),
+         float(q_scale), _ptr(state), _ptr(ctx.state_slots), _ptr(ctx.cu_tokens), _ptr(out), ctx.n_entries,
          nh, dk, dv, _stream())
     return out
 

@@ -15,7 +15,8 @@ class GatedLinearAttention(Part):
     """Linear attention with a decay per key channel.  With h the input, per head (dk key
     channels, dv value channels): q = W_q h * dk^(-1/2), k = W_k h, v = W_v h, and a decay
     alpha = sigmoid(z)^(1/tau) in (0, 1) for every key channel, z = W_a2 (W_a1 h) + b through a
-    narrow middle (``decay_rank``).  The state S [dk, dv] starts at zero and moves token by token,
+    narrow middle (``decay_rank``; in steps of few tokens W_a2, the bias and the decay itself are
+    one kernel).  The state S [dk, dv] starts at zero and moves token by token,
     S_t = diag(alpha_t) S_(t-1) + k_t v_t^T; the head's output is o_t = S_t^T q_t, RMS-normed over
     dv with learned weights shared by the heads; the heads side by side are multiplied by
     silu(W_g h) and projected by W_o.
@@ -26,6 +27,7 @@ class GatedLinearAttention(Part):
     in order from the slot's state (csrc/linear_attention.hip), so the outputs of a token do not
     depend on how its request was cut into steps."""
 
+    FUSED_DECAY_TOKENS = 64    # up to so many tokens a step, W_a2, the bias and the decay are one kernel
     NAMES = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o", "norm": "norm", "a1": "a1", "a2": "a2", "a2_bias": "a2.b"}
 
     def __init__(self, hidden: int, num_heads: int, key_dim: int, value_dim: int, tau: float, decay_rank: int,
@@ -41,8 +43,8 @@ class GatedLinearAttention(Part):
         self.names = {**self.NAMES, **(names or {})}
         self.graph_safe = True         # entries and their state slots are read from the step's device arrays
         self.w_in = None               # [q | k | v | g] rows: one product of the input
-        self.w_a1 = None
-        self.w_a2 = None
+        self.w_a1 = None               # (a product of its own: a few rows more spoil the large product's shape)
+        self.w_a2: Optional[torch.Tensor] = None      # [heads * dk, rank], row-major
         self.b_a2: Optional[torch.Tensor] = None      # float32 [heads * dk]
         self.w_norm: Optional[torch.Tensor] = None    # float32 [dv]
         self.w_o = None
@@ -77,7 +79,7 @@ class GatedLinearAttention(Part):
             o += p.shape[0]
         self.w_in = ops.pack_weight(fused)
         self.w_a1 = ops.pack_weight(source.get(prefix + n["a1"]))
-        self.w_a2 = ops.pack_weight(source.get(prefix + n["a2"]))
+        self.w_a2 = source.get(prefix + n["a2"]).to(dt).contiguous()
         self.b_a2 = source.get(prefix + n["a2_bias"]).float().contiguous()
         self.w_norm = source.get(prefix + n["norm"]).float().contiguous()
         self.w_o = ops.pack_weight(source.get(prefix + n["o"]))
@@ -91,13 +93,16 @@ class GatedLinearAttention(Part):
         n_in = 2 * qk + (2 if self.has_gate else 1) * vv
         with section("q|k|v|g", nbytes=width * n_in * (self.hidden + T) + width * T * self.hidden, flops=2.0 * T * self.hidden * n_in):
             proj = ops.linear(x, self.w_in, ctx.act_dtype)
-        with section("decay logits", nbytes=width * self.rank * (self.hidden + qk) + 4 * T * qk,
-                     flops=2.0 * T * self.rank * (self.hidden + qk)):
-            z = ops.linear(ops.linear(x, self.w_a1, ctx.act_dtype), self.w_a2, torch.float32)
+        with section("decays", nbytes=width * self.rank * (self.hidden + T + qk) + 4 * T * qk, flops=2.0 * T * self.rank * (self.hidden + qk)):
+            a1 = ops.linear(x, self.w_a1, ctx.act_dtype)
+            if T <= self.FUSED_DECAY_TOKENS and self.rank <= ops.GLA_FUSED_DECAY_MAX_RANK and a1.dtype == self.w_a2.dtype:
+                alpha = ops.gla_decays_from_middle(a1, 0, self.rank, self.w_a2, self.b_a2, self.tau)     # few tokens: one kernel
+            else:
+                alpha = ops.gla_decays(ops.linear(a1, self.w_a2, torch.float32), self.b_a2, self.tau)
         state = cache.states[0] if cache.states else cache.state
         with section("recurrence", nbytes=lambda: 8 * ctx.n_entries * qk * self.dv + T * (width * (2 * qk + vv) + 4 * (qk + vv)),
                      flops=4.0 * T * qk * self.dv):
-            o = ops.gla_walk(proj, 0, qk, 2 * qk, z, self.b_a2, self.tau, self.dk ** -0.5, state, ctx, self.nh, self.dk, self.dv)
+            o = ops.gla_walk(proj, 0, qk, 2 * qk, alpha, self.dk ** -0.5, state, ctx, self.nh, self.dk, self.dv)
         with section("head norm + gate", nbytes=T * vv * (4 + 2 * width)):
             y = ops.head_norm_gate(o, self.w_norm, self.eps, self.nh, self.dv, ctx.act_dtype,
                                    proj if self.has_gate else None, 2 * qk + vv)

@@ -158,7 +158,7 @@ def test_the_recurrence_walks_every_entry_from_its_slots_state(dtype, H, dk, dv,
 
     g = torch.Generator().manual_seed(dk + dv)
     qk, vv = H * dk, H * dv
-    pad = 3
+    pad = 3 if dk % 16 else 8                                    # (rows of eight aligned elements take the wide loads)
     plan = [[("a", 1), ("b", 40)], [("b", 1), ("c", 7), ("a", 2)], [("a", 9), ("c", 1)]]
     total = {"a": 12, "b": 41, "c": 8}
     slot_of = {"a": 3, "b": 0, "c": 1}
@@ -173,7 +173,9 @@ def test_the_recurrence_walks_every_entry_from_its_slots_state(dtype, H, dk, dv,
         ctx = _Step([n for _, n in step], [at[r] for r, _ in step], [slot_of[r] for r, _ in step])
         rows = torch.cat([proj[r][at[r]:at[r] + n] for r, n in step]).to(DEV)
         zz = torch.cat([z[r][at[r]:at[r] + n] for r, n in step]).to(DEV)
-        o = ops.gla_walk(rows, pad, pad + qk, pad + 2 * qk, zz, bias.to(DEV), tau, dk ** -0.5, state, ctx, H, dk, dv)
+        decays = ops.gla_decays(zz, bias.to(DEV), tau)
+        assert decays.data_ptr() == zz.data_ptr()              # made in place over the logits
+        o = ops.gla_walk(rows, pad, pad + qk, pad + 2 * qk, decays, dk ** -0.5, state, ctx, H, dk, dv)
         i = 0
         for r, n in step:
             got[r].append(o[i:i + n].cpu())
@@ -186,6 +188,24 @@ def test_the_recurrence_walks_every_entry_from_its_slots_state(dtype, H, dk, dv,
                                   p[:, pad + 2 * qk:].reshape(n, H, dv), alpha)
         assert _rel_rms(torch.cat(got[r]), want.reshape(n, -1)) < 2e-6, r      # float arithmetic in both dtypes
     assert float((state[2] - 9.0).abs().max()) == 0.0 and float(state[4].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("T, N, rank, tau", [(1, 20, 5, 3.0), (19, 288, 16, 16.0), (70, 520, 64, 0.5), (9, 40, 256, 1.0)])
+def test_decays_from_the_narrow_middle_of_their_projection(dtype, T, N, rank, tau):
+    from sharpinference_amd import ops
+
+    g = torch.Generator().manual_seed(T + rank)
+    pad = 11
+    proj = torch.randn(T, pad + rank + 2, generator=g).to(DT[dtype])
+    w = torch.randn(N, rank, generator=g).to(DT[dtype])
+    bias = torch.randn(N, generator=g) * 2
+    got = ops.gla_decays_from_middle(proj.to(DEV), pad, rank, w.to(DEV), bias.to(DEV), tau)
+    z = proj.double()[:, pad:pad + rank] @ w.double().T + bias.double()
+    want = torch.exp(torch.nn.functional.logsigmoid(z) / tau)
+    assert got.dtype == torch.float32 and float((got.cpu().double() - want).abs().max()) < 2e-6     # decays lie in (0, 1)
+    two = ops.gla_decays((proj[:, pad:pad + rank].float() @ w.float().T).to(DEV), bias.to(DEV), tau)   # the two-kernel form
+    assert float((two.cpu().double() - want).abs().max()) < 1e-5
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
