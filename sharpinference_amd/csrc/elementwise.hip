@@ -534,3 +534,86 @@ SHARPI_EXPORT int sharpi_norm_mean(const void* const* xs, const float* const* ws
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }
+
+// ---------------------------------------------------------------------------
+// The norm behind a branch and the norm before the next one, in one pass over a row:
+//   y   = the branch's output (a tensor; or the join of side-by-side branches, formed here as norm_mean does)
+//   h  += unit_rms(y) * w_post                       (the float residual sum, in place)
+//   out = unit_rms(h) * w_next  (if asked for)       (what the next branch reads)
+// One block a row; the row stays in LDS (float) between the passes; statistics and sums in float.
+// ---------------------------------------------------------------------------
+template <typename TD, typename TO>
+__global__ __launch_bounds__(256) void post_pre_norm_kernel(float* __restrict__ h, BranchArgs a, int n_branches,
+                                                            const float* __restrict__ w_post, const float* __restrict__ w_next,
+                                                            TO* __restrict__ out, int N, float eps) {
+  extern __shared__ float yrow[];
+  __shared__ float red[16];
+  const size_t t = blockIdx.x;
+  if (n_branches == 1 && a.w[0] == nullptr) {
+    const TD* x = (const TD*)a.x[0] + t * N;
+    for (int i = threadIdx.x; i < N; i += blockDim.x) yrow[i] = to_f32<TD>(x[i]);
+  } else {
+    float inv[kMaxBranches];
+    for (int b = 0; b < n_branches; ++b) {
+      const TD* x = (const TD*)a.x[b] + t * N;
+      float ss = 0.f;
+      for (int i = threadIdx.x; i < N; i += blockDim.x) {
+        const float v = to_f32<TD>(x[i]);
+        ss = fmaf(v, v, ss);
+      }
+      inv[b] = rsqrtf(block_sum(ss, red) / (float)N + eps);
+    }
+    const float share = 1.0f / (float)n_branches;
+    for (int i = threadIdx.x; i < N; i += blockDim.x) {
+      float y = 0.f;
+      for (int b = 0; b < n_branches; ++b) y += to_f32<TD>(((const TD*)a.x[b])[t * N + i]) * inv[b] * a.w[b][i];
+      yrow[i] = y * share;
+    }
+  }
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < N; i += blockDim.x) ss = fmaf(yrow[i], yrow[i], ss);   // (a thread reads what it wrote)
+  const float inv_y = rsqrtf(block_sum(ss, red) / (float)N + eps);
+  float* hr = h + t * N;
+  float s2 = 0.f;
+  for (int i = threadIdx.x; i < N; i += blockDim.x) {
+    const float v = hr[i] + yrow[i] * inv_y * w_post[i];
+    hr[i] = v;
+    yrow[i] = v;
+    s2 = fmaf(v, v, s2);
+  }
+  if (!out) return;
+  const float inv_h = rsqrtf(block_sum(s2, red) / (float)N + eps);
+  for (int i = threadIdx.x; i < N; i += blockDim.x) out[t * N + i] = from_f32<TO>(yrow[i] * inv_h * w_next[i]);
+}
+
+// h float [T, N] in place; xs: n_branches tensors [T, N] of `d_dtype`, ws: their float weights [N] (ws[0] null with one
+// branch: the tensor itself is the branch output); w_post float [N]; out [T, N] of `o_dtype` with w_next float [N], or null.
+SHARPI_EXPORT int sharpi_post_pre_norm(float* h, const void* const* xs, const float* const* ws, int n_branches, int d_dtype,
+                                       const float* w_post, const float* w_next, void* out, int o_dtype, int n_rows, int N,
+                                       float eps, hipStream_t stream) {
+  if (n_rows <= 0) return SHARPI_OK;
+  if (n_branches < 1 || n_branches > kMaxBranches || N <= 0 || !w_post || (out && !w_next)) return SHARPI_ERR_ARG;
+  if ((size_t)N * sizeof(float) > 60 * 1024) return SHARPI_ERR_ARG;
+  BranchArgs a{};
+  for (int b = 0; b < n_branches; ++b) {
+    if (!xs[b] || (!ws[b] && n_branches > 1)) return SHARPI_ERR_ARG;
+    a.x[b] = xs[b];
+    a.w[b] = ws[b];
+  }
+  const size_t lds = (size_t)N * sizeof(float);
+#define PPN(TD, TO) post_pre_norm_kernel<TD, TO><<<n_rows, 256, lds, stream>>>(h, a, n_branches, w_post, w_next, (TO*)out, N, eps)
+  const bool of = !out || o_dtype == DT_F32;
+  if (out && o_dtype != DT_F32 && o_dtype != DT_BF16) return SHARPI_ERR_ARG;
+  if (d_dtype == DT_F32) {
+    if (of) PPN(float, float);
+    else PPN(float, bf16_t);
+  } else if (d_dtype == DT_BF16) {
+    if (of) PPN(bf16_t, float);
+    else PPN(bf16_t, bf16_t);
+  } else {
+    return SHARPI_ERR_ARG;
+  }
+#undef PPN
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}

@@ -1,7 +1,11 @@
 // Gated linear attention: a matrix-valued recurrent state per head with a decay per key channel,
 //   S_t = diag(alpha_t) S_(t-1) + k_t v_t^T,   o_t = S_t^T q_t,   alpha_t = sigmoid(z_t)^(1/tau),
-// walked token by token in float.  The state of a request lives in its state slot
-// [slots, heads, dk, dv] (float) and is carried from step to step.
+// walked token by token in float.  The state of a request lives in its state slot and is carried
+// from step to step.  It is kept column slice by column slice, [slots, heads, ceil(dv / 8), dk, 8]
+// (float): the 8 columns a block owns are then one contiguous piece of memory, which the block
+// alone reads and writes (row-major [dk, dv], a block's 32 bytes of every row would share their
+// cache lines with three other blocks on other compute dies, and every line would cross the
+// memory interface four times).
 //
 // A block owns kCols value columns of one head of one entry: the columns of S are independent of
 // each other, so an entry's work is spread over heads x ceil(dv / kCols) blocks, and the walk along
@@ -84,13 +88,13 @@ __global__ __launch_bounds__(2 * kWave) void gla_walk_kernel(
   const int col = c0 + j;
   const bool col_ok = col < dv;
   const int first = cu_tokens[e], len = cu_tokens[e + 1] - first;
-  float* S = state + (((size_t)state_slots[e] * nh + h) * dk) * dv;
+  float* S = state + ((((size_t)state_slots[e] * nh + h) * gridDim.x + blockIdx.x) * dk) * kCols;
   float s[RPL];
   if (walker) {
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
       const int rowi = g * RPL + r;
-      s[r] = (col_ok && rowi < dk) ? S[(size_t)rowi * dv + col] : 0.f;
+      s[r] = (col_ok && rowi < dk) ? S[(size_t)rowi * kCols + j] : 0.f;
     }
   }
   auto stage = [&](int t0, int buf) {
@@ -193,7 +197,7 @@ __global__ __launch_bounds__(2 * kWave) void gla_walk_kernel(
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
       const int rowi = g * RPL + r;
-      if (col_ok && rowi < dk) S[(size_t)rowi * dv + col] = s[r];
+      if (col_ok && rowi < dk) S[(size_t)rowi * kCols + j] = s[r];
     }
   }
 }
@@ -252,6 +256,9 @@ static int launch_walk(const void* proj, int stride, int q_off, int k_off, int v
 }
 
 // z float [n_rows, N]: decay logits, turned in place into decays sigmoid(z + bias)^(1 / tau), bias [N].
+// columns of the state that lie together in memory (the state's layout is [.., ceil(dv / this), dk, this])
+SHARPI_EXPORT int sharpi_gla_state_cols() { return kCols; }
+
 SHARPI_EXPORT int sharpi_gla_decays(float* z, const float* bias, float tau, int n_rows, int N, hipStream_t stream) {
   if (n_rows <= 0) return SHARPI_OK;
   if (N <= 0 || !(tau > 0.f) || !bias) return SHARPI_ERR_ARG;
@@ -284,7 +291,7 @@ SHARPI_EXPORT int sharpi_gla_decays_fused(const void* proj, int dtype, int strid
 }
 
 // proj [T, stride] of `dtype` holds q (nh * dk columns at q_off), k (at k_off) and v (nh * dv at
-// v_off); alpha float [T, nh * dk] are the decays; state float [slots, nh, dk, dv]; out float
+// v_off); alpha float [T, nh * dk] are the decays; state float [slots, nh, ceil(dv / 8), dk, 8]; out float
 // [T, nh * dv].  Entries (cu_tokens [entries + 1]) are walked in parallel, each from the state of
 // its slot, which is left advanced.
 SHARPI_EXPORT int sharpi_gla_walk(const void* proj, int dtype, int stride, int q_off, int k_off, int v_off,

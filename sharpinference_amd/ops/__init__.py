@@ -1184,6 +1184,20 @@ def qk_prep(proj: torch.Tensor, q_off: int, k_off: int, v_off: Optional[int], nh
 # gated linear attention
 # ---------------------------------------------------------------------------
 GLA_MAX_KEY_DIM = 256      # key channels of a head that the walk holds (csrc/linear_attention.hip)
+GLA_STATE_COLS = _lib.GLA_STATE_COLS   # value columns of the state that lie together in memory (checked against the library at load)
+
+
+def gla_state_shape(nh: int, dk: int, dv: int) -> tuple:
+    """A request's recurrent state as the walk keeps it: [heads, ceil(dv / 8), dk, 8], column slice by
+    column slice (element (h, i, j) of the matrices S_h [dk, dv] lies at [h, j // 8, i, j % 8])."""
+    return (nh, (dv + GLA_STATE_COLS - 1) // GLA_STATE_COLS, dk, GLA_STATE_COLS)
+
+
+def gla_state_matrices(state: torch.Tensor, dv: int) -> torch.Tensor:
+    """[.., heads, ceil(dv / 8), dk, 8] as kept -> the matrices [.., heads, dk, dv] (a copy; for tests and tools)."""
+    *lead, nh, ncb, dk, c = state.shape
+    return state.movedim(-3, -2).reshape(*lead, nh, dk, ncb * c)[..., :dv].contiguous()
+
 
 
 def gla_decays(z: torch.Tensor, bias: torch.Tensor, tau: float) -> torch.Tensor:
@@ -1219,8 +1233,8 @@ def gla_decays_from_middle(proj: torch.Tensor, a_off: int, rank: int, w: torch.T
 def gla_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, alpha: torch.Tensor, q_scale: float,
              state: torch.Tensor, ctx, nh: int, dk: int, dv: int) -> torch.Tensor:
     """The recurrence S_t = diag(alpha_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per head, token by
-    token along every entry of the step, from and into state [slots, nh, dk, dv] (float32) at the
-    entries' state slots.  q, k (nh*dk columns each) and v (nh*dv) are columns of proj [T, N]; q is
+    token along every entry of the step, from and into state [slots, *gla_state_shape(nh, dk, dv)]
+    (float32) at the entries' state slots.  q, k (nh*dk columns each) and v (nh*dv) are columns of proj [T, N]; q is
     multiplied by q_scale; alpha float32 [T, nh*dk] are the decays.  Returns o float32 [T, nh*dv]."""
     _dev(proj, alpha, state)
     T, N = proj.shape
@@ -1228,8 +1242,8 @@ def gla_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, alpha: torc
     _need(min(q_off, k_off, v_off) >= 0 and max(q_off, k_off) + nh * dk <= N and v_off + nh * dv <= N,
           "gla_walk: q, k and v columns must lie inside proj")
     _need(alpha.dtype == torch.float32 and alpha.shape == (T, nh * dk), "gla_walk: alpha float32 [T, nh*dk] wanted")
-    _need(state.dtype == torch.float32 and state.dim() == 4 and tuple(state.shape[1:]) == (nh, dk, dv),
-          "gla_walk: state must be float32 [slots, nh, dk, dv]")
+    _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == gla_state_shape(nh, dk, dv),
+          "gla_walk: state must be float32 [slots, nh, ceil(dv / 8), dk, 8]")
     _need(ctx.state_slots.shape == (ctx.n_entries,) and ctx.cu_tokens.shape == (ctx.n_entries + 1,) and ctx.n_tokens == T,
           "gla_walk: the step's per-entry arrays do not fit")
     out = torch.empty(T, nh * dv, dtype=torch.float32, device=proj.device)
@@ -1255,6 +1269,54 @@ def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, eps: float, nh: int, d
     out = torch.empty(T, nh * dv, dtype=out_dtype, device=o.device)
     _run("sharpi_head_norm_gate", _ptr(o), _ptr(weight), float(eps), _ptr(gate_proj), _code(out_dtype), stride, int(gate_off),
          _ptr(out), T, nh, dv, _stream())
+    return out
+
+
+class BranchMean:
+    """Stands for the join of side-by-side branches, (1 / n) * sum_b unit_rms(xs[b]) * weights[b], still to
+    be formed: float32 [T, N].  The norm kernel behind the branches forms it while it reads them
+    (:func:`post_pre_norm`); ``tensor()`` forms it on its own for whoever needs a tensor."""
+
+    def __init__(self, xs, weights, eps: float):
+        self.xs, self.weights, self.eps = list(xs), list(weights), float(eps)
+        self.shape, self.dtype = tuple(xs[0].shape), torch.float32
+
+    def tensor(self) -> torch.Tensor:
+        return norm_mean(self.xs, self.weights, self.eps)
+
+
+POST_PRE_NORM_MAX_WIDTH = 15 * 1024     # floats of a row that the kernel keeps in LDS
+
+
+def post_pre_norm(h: torch.Tensor, delta, w_post: torch.Tensor, eps: float, w_next: Optional[torch.Tensor] = None,
+                  out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """h += unit_rms(delta) * w_post in place in float, and, with w_next, returns unit_rms(new h) *
+    w_next in out_dtype: the norm behind one branch and the norm before the next in one launch.
+    delta: a tensor [T, N] or a BranchMean (formed by the kernel, with the eps of its own it was
+    made with, which must equal eps).  Weights float32 [N]."""
+    import ctypes
+
+    lazy = delta if isinstance(delta, BranchMean) else None
+    xs = lazy.xs if lazy is not None else [delta]
+    ws = lazy.weights if lazy is not None else [None]
+    _dev(h, w_post, w_next, *xs, *[w for w in ws if w is not None])
+    _need(h.dim() == 2 and h.dtype == torch.float32, "post_pre_norm: h must be float32 [T, N]")
+    T, N = h.shape
+    _need(N <= POST_PRE_NORM_MAX_WIDTH and 1 <= len(xs) <= NORM_MEAN_MAX_BRANCHES, "post_pre_norm: row too wide or too many branches")
+    _need(lazy is None or lazy.eps == float(eps), "post_pre_norm: the join was made with another eps")
+    for x, w in zip(xs, ws):
+        _need(tuple(x.shape) == (T, N) and x.dtype == xs[0].dtype and (w is None or (w.dtype == torch.float32 and w.shape == (N,))),
+              "post_pre_norm: branches [T, N] of one dtype, weights float32 [N]")
+    _need(w_post.dtype == torch.float32 and w_post.shape == (N,), "post_pre_norm: w_post must be float32 [N]")
+    out = None
+    if w_next is not None:
+        _need(w_next.dtype == torch.float32 and w_next.shape == (N,) and out_dtype is not None, "post_pre_norm: w_next float32 [N] and an out_dtype")
+        out = torch.empty(T, N, dtype=out_dtype, device=h.device)
+    n = len(xs)
+    xp = (ctypes.c_void_p * n)(*[x.data_ptr() for x in xs])
+    wp = (ctypes.c_void_p * n)(*[(w.data_ptr() if w is not None else None) for w in ws])
+    _run("sharpi_post_pre_norm", _ptr(h), ctypes.cast(xp, ctypes.c_void_p), ctypes.cast(wp, ctypes.c_void_p), n, _code(xs[0].dtype),
+         _ptr(w_post), _ptr(w_next), _ptr(out), _code(out_dtype) if out is not None else 0, T, N, float(eps), _stream())
     return out
 
 

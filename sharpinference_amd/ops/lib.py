@@ -56,6 +56,7 @@ _SIGNATURES = {
     "sharpi_head_norm_gate": [P, P, F, P, I, I, I, P, I, I, I, P],
     "sharpi_activation": [P, P, I, c_longlong, I, P],
     "sharpi_norm_mean": [P, P, I, I, P, I, I, F, P],
+    "sharpi_post_pre_norm": [P, P, P, I, I, P, P, P, I, I, I, F, P],
 }
 
 # entry points that newer sources add; bound when present
@@ -68,12 +69,14 @@ PREFILL_TILE_TOKENS = 128   # tokens per block of the prefill attention kernel
 PICKED_MAX_PAIRS = 64       # (token, pick) pairs the few-rows product takes straight from the router's picks
 FUSED_NORM_ROUTER_MAX_HIDDEN = 8192   # widest row of the norm + router kernel
 ROUTER_MAX_EXPERTS = 1024   # experts the routing kernels hold scores for
+GLA_STATE_COLS = 8          # value columns of a linear-attention state that lie together in memory
 _BUILT_WITH = {
     "sharpi_attention_decode_split_keys": DECODE_RUN_KEYS,
     "sharpi_attention_prefill_tile_tokens": PREFILL_TILE_TOKENS,
     "sharpi_router_max_experts": ROUTER_MAX_EXPERTS,
     "sharpi_gemm_skinny_max_picked": PICKED_MAX_PAIRS,
     "sharpi_add_rmsnorm_router_max_hidden": FUSED_NORM_ROUTER_MAX_HIDDEN,
+    "sharpi_gla_state_cols": GLA_STATE_COLS,
 }
 
 

@@ -127,7 +127,16 @@ class ResidualStream:
     def __init__(self, h: torch.Tensor):
         self.h = h
         self.pending = None
+        self.pending_norm = None   # a norm that sits on `pending` before it is added (h += norm(pending)): the norm
+                                   # part that folds both into the next norm's launch, or `settle()`, applies it
         self.act = None        # h in the activations' storage type, where a block keeps such a copy beside it
+
+    def settle(self) -> None:
+        """Add a branch output that waits behind a norm of its own into the sum now."""
+        if self.pending_norm is not None:
+            norm, delta = self.pending_norm, self.pending
+            self.pending = self.pending_norm = None
+            norm.add_normed(self, delta, None)
 
     def pending_tensor(self) -> Optional[torch.Tensor]:
         p = self.pending

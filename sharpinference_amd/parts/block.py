@@ -85,6 +85,7 @@ class PostNormBlock(PreNormBlock):
 
     @staticmethod
     def _input(stream: ResidualStream, ctx: StepContext) -> torch.Tensor:
+        stream.settle()
         if stream.pending is not None:
             raise ValueError("a block with norms on its outputs cannot follow one that leaves its output pending")
         if stream.act is None or stream.act.dtype != ctx.act_dtype:
@@ -101,8 +102,10 @@ class PostNormBlock(PreNormBlock):
 
 class SandwichBlock(PreNormBlock):
     """h += norm1b(mixer(norm1(h))); h += norm2b(ffn(norm2(h))): a norm before and a norm after each
-    branch.  ``ffn`` None: a layer of a mixer alone.  Nothing is left pending: the norm behind a
-    branch adds into the float residual sum itself."""
+    branch.  ``ffn`` None: a layer of a mixer alone.  The norm behind a branch and the norm before
+    the next branch are one launch (``RMSNorm.after``); the block's last branch output is left
+    waiting behind its norm (``stream.pending_norm``) for the next block's first norm, or for
+    whoever settles the stream."""
 
     def __init__(self, norm1: Part, mixer: Part, norm1b: Part, norm2: Part = None, ffn: Part = None, norm2b: Part = None,
                  names=None):
@@ -119,8 +122,10 @@ class SandwichBlock(PreNormBlock):
         return tuple(kids)
 
     def forward(self, stream: ResidualStream, ctx: StepContext, cache: LayerCache) -> None:
-        n = self.norm1.forward(stream, ctx.act_dtype)           # (folds in what a block before may have left pending)
-        self.norm1b.add_normed(stream, self.mixer.forward(n, ctx, cache), None)
-        if self.ffn is not None:
-            n = self.norm2.forward(stream, ctx.act_dtype)
-            self.norm2b.add_normed(stream, self.ffn.forward(n, ctx), None)
+        n = self.norm1.forward(stream, ctx.act_dtype)           # (with the norm behind the branch a block before left waiting)
+        y = self.mixer.forward(n, ctx, cache)
+        if self.ffn is None:
+            stream.pending, stream.pending_norm = y, self.norm1b    # waits for the next norm's launch (or `settle`)
+            return
+        n = self.norm2.after(self.norm1b, stream, y, ctx.act_dtype)
+        stream.pending, stream.pending_norm = self.ffn.forward(n, ctx), self.norm2b

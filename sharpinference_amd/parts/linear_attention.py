@@ -21,8 +21,8 @@ class GatedLinearAttention(Part):
     dv with learned weights shared by the heads; the heads side by side are multiplied by
     silu(W_g h) and projected by W_o.
 
-    What is kept per request is the state alone, [heads, dk, dv] in float, in the request's state
-    slot: no pages.  Decays (their logarithm, the division by tau, the exponential), the state and
+    What is kept per request is the state alone, heads x dk x dv floats in the request's state
+    slot (laid out column slice by column slice, ``ops.gla_state_shape``): no pages.  Decays (their logarithm, the division by tau, the exponential), the state and
     the norm are float whatever the activations are stored as.  A step walks each entry's tokens
     in order from the slot's state (csrc/linear_attention.hip), so the outputs of a token do not
     depend on how its request was cut into steps."""
@@ -50,7 +50,7 @@ class GatedLinearAttention(Part):
         self.w_o = None
 
     def cache_spec(self) -> StateSpec:
-        return StateSpec((self.nh, self.dk, self.dv), torch.float32)
+        return StateSpec(ops.gla_state_shape(self.nh, self.dk, self.dv), torch.float32)
 
     def param_specs(self, prefix: str) -> Dict[str, ParamSpec]:
         n, qk, vv = self.names, self.nh * self.dk, self.nh * self.dv

@@ -144,6 +144,7 @@ class DecoderModel(Part):
         for r in self.schedule:
             c = caches[r.cache]
             if r.add_row is not None:
+                stream.settle()
                 if stream.pending is not None:
                     raise ValueError("a row can be added only where no branch output is pending")
                 with section("row added to the stream", nbytes=ctx.n_tokens * self.hidden * 8):

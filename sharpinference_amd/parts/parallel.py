@@ -19,8 +19,8 @@ class ParallelMixers(Part):
     ``branches``: (name, mixer) pairs; branch b's tensors lie under ``<prefix><name>.`` and its norm
     weight is ``<prefix><name>.<out_name>``.  At most one branch may keep pages; the fixed-size
     states of all of them are asked for together and handed back to each in its own order.  The
-    join is float (statistics, weights, the sum) and leaves a float tensor for the norm or the
-    addition that follows."""
+    join is float (statistics, weights, the sum); ``forward`` returns it as an ``ops.BranchMean``, which
+    the norm kernel behind the mixer forms itself (``tensor()`` forms it for anyone else)."""
 
     def __init__(self, hidden: int, branches: Sequence[Tuple[str, Part]], norm_eps: float, out_name: str = "out"):
         if not 1 <= len(branches) <= ops.NORM_MEAN_MAX_BRANCHES:
@@ -68,5 +68,5 @@ class ParallelMixers(Part):
             sub = LayerCache(group=cache.group if has_pages else None, k=cache.k if has_pages else None,
                              v=cache.v if has_pages else None, state=mine[0] if mine else None, write=cache.write, states=mine)
             outs.append(m.forward(x, ctx, sub))
-        with section("join of the branches", nbytes=x.shape[0] * self.hidden * (4 + len(outs) * outs[0].element_size())):
-            return ops.norm_mean(outs, self.w_out, self.eps)
+        # the join is left to the norm kernel that follows, which forms it while it reads the branches
+        return ops.BranchMean(outs, self.w_out, self.eps)

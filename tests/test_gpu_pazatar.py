@@ -165,7 +165,7 @@ def test_the_recurrence_walks_every_entry_from_its_slots_state(dtype, H, dk, dv,
     proj = {r: torch.randn(n, pad + 2 * qk + vv, generator=g).to(DT[dtype]) for r, n in total.items()}
     z = {r: torch.randn(n, qk, generator=g) * 2 for r, n in total.items()}
     bias = torch.randn(qk, generator=g)
-    state = torch.zeros(5, H, dk, dv, device=DEV)
+    state = torch.zeros(5, *ops.gla_state_shape(H, dk, dv), device=DEV)
     state[2].fill_(9.0)                                          # a slot no entry names
     got = {r: [] for r in total}
     at = {r: 0 for r in total}
@@ -188,6 +188,16 @@ def test_the_recurrence_walks_every_entry_from_its_slots_state(dtype, H, dk, dv,
                                   p[:, pad + 2 * qk:].reshape(n, H, dv), alpha)
         assert _rel_rms(torch.cat(got[r]), want.reshape(n, -1)) < 2e-6, r      # float arithmetic in both dtypes
     assert float((state[2] - 9.0).abs().max()) == 0.0 and float(state[4].abs().max()) == 0.0
+    # what the slots hold in the end are the matrices S of the plain recurrence: sum_s (prod of later decays) k_s v_s^T
+    for r, n in total.items():
+        p = proj[r].double()
+        alpha = torch.exp(torch.nn.functional.logsigmoid(z[r].double() + bias.double()) / tau).reshape(n, H, dk)
+        k, v = p[:, pad + qk:pad + 2 * qk].reshape(n, H, dk), p[:, pad + 2 * qk:].reshape(n, H, dv)
+        S = torch.zeros(H, dk, dv, dtype=torch.float64)
+        for t in range(n):
+            S = alpha[t][:, :, None] * S + k[t][:, :, None] * v[t][:, None, :]
+        got_S = ops.gla_state_matrices(state[slot_of[r]], dv).cpu()
+        assert _rel_rms(got_S.reshape(1, -1), S.reshape(1, -1)) < 2e-6, f"state of {r}"
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -231,6 +241,39 @@ def test_head_norm_with_gate_the_join_of_branches_and_the_squared_relu(dtype):
     assert _rel_rms(ops.norm_mean([a.to(DEV)], [wa.to(DEV)], 1e-5), P.rms_norm(a.double(), wa.double(), 1e-5)) < 2e-6
     x = torch.randn(T, 50, generator=g).to(DT[dtype])
     assert _rel_rms(ops.activation(x.to(DEV), "relu2"), P.relu_squared(x.double())) < tol
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("T, N", [(1, 72), (9, 320), (70, 2048)])
+def test_the_norm_behind_a_branch_and_the_norm_before_the_next_in_one_launch(dtype, T, N):
+    from sharpinference_amd import ops
+
+    g = torch.Generator().manual_seed(T + N)
+    h = torch.randn(T, N, generator=g) * 3
+    y = (torch.randn(T, N, generator=g) * 0.2).to(DT[dtype])
+    a, b = (torch.randn(T, N, generator=g) * 5).to(DT[dtype]), (torch.randn(T, N, generator=g) * 0.3).to(DT[dtype])
+    wp, wn, wa, wb = (0.5 + torch.rand(N, generator=g) for _ in range(4))
+    eps = 1e-5
+    tol = 2e-6 if dtype == "float32" else 6e-3
+    # one branch, with and without the next norm
+    hd = h.to(DEV)
+    out = ops.post_pre_norm(hd, y.to(DEV), wp.to(DEV), eps, wn.to(DEV), DT[dtype])
+    want_h = h.double() + P.rms_norm(y.double(), wp.double(), eps)
+    assert _rel_rms(hd, want_h) < 2e-6 and out.dtype == DT[dtype]
+    assert _rel_rms(out, P.rms_norm(want_h, wn.double(), eps)) < tol
+    hd2 = h.to(DEV)
+    assert ops.post_pre_norm(hd2, y.to(DEV), wp.to(DEV), eps) is None and torch.equal(hd2, hd)
+    hd3 = h.to(DEV)
+    ops.norm_add(hd3, y.to(DEV), wp.to(DEV), eps, None)                       # the unfused kernel: the same sum
+    assert _rel_rms(hd3, hd.cpu()) < 1e-6
+    # the join of two branches formed on the way
+    hd = h.to(DEV)
+    join = ops.BranchMean([a.to(DEV), b.to(DEV)], [wa.to(DEV), wb.to(DEV)], eps)
+    out = ops.post_pre_norm(hd, join, wp.to(DEV), eps, wn.to(DEV), DT[dtype])
+    mean = 0.5 * (P.rms_norm(a.double(), wa.double(), eps) + P.rms_norm(b.double(), wb.double(), eps))
+    want_h = h.double() + P.rms_norm(mean, wp.double(), eps)
+    assert _rel_rms(join.tensor(), mean) < 2e-6
+    assert _rel_rms(hd, want_h) < 2e-6 and _rel_rms(out, P.rms_norm(want_h, wn.double(), eps)) < tol
 
 
 class _Ctx:
