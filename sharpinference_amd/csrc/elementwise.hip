@@ -1,6 +1,7 @@
 // Row-wise kernels: embedding gather, residual add + RMSNorm, SiLU*up, MoE combine, casts.
 // All statistics and sums are float; storage may be float or bfloat16.
 #include "common.h"
+#include <type_traits>
 
 // ---------------------------------------------------------------------------
 // embedding gather: out[t, :] = table[ids[t], :] * scale   (out is the float residual stream; the
@@ -542,48 +543,86 @@ SHARPI_EXPORT int sharpi_norm_mean(const void* const* xs, const float* const* ws
 //   out = unit_rms(h) * w_next  (if asked for)       (what the next branch reads)
 // One block a row; the row stays in LDS (float) between the passes; statistics and sums in float.
 // ---------------------------------------------------------------------------
-template <typename TD, typename TO>
+template <typename TD, typename TO, int V>     // V: elements a thread takes at a time (8 where N is a multiple of 8, else 1)
 __global__ __launch_bounds__(256) void post_pre_norm_kernel(float* __restrict__ h, BranchArgs a, int n_branches,
                                                             const float* __restrict__ w_post, const float* __restrict__ w_next,
                                                             TO* __restrict__ out, int N, float eps) {
-  extern __shared__ float yrow[];
+  extern __shared__ __attribute__((aligned(16))) float yrow[];
   __shared__ float red[16];
   const size_t t = blockIdx.x;
+  const int step = blockDim.x * V;
+  auto get = [](const auto* p, float* v) {
+    if constexpr (V == 8) load8(p, v);
+    else v[0] = to_f32<std::remove_cv_t<std::remove_reference_t<decltype(*p)>>>(*p);
+  };
+  auto put = [](auto* p, const float* v) {
+    if constexpr (V == 8) store8(p, v);
+    else *p = from_f32<std::remove_reference_t<decltype(*p)>>(v[0]);
+  };
+  float x[V], w[V], y[V];
   if (n_branches == 1 && a.w[0] == nullptr) {
-    const TD* x = (const TD*)a.x[0] + t * N;
-    for (int i = threadIdx.x; i < N; i += blockDim.x) yrow[i] = to_f32<TD>(x[i]);
+    const TD* xr = (const TD*)a.x[0] + t * N;
+    for (int i = threadIdx.x * V; i < N; i += step) {
+      get(xr + i, x);
+      put(yrow + i, x);
+    }
   } else {
     float inv[kMaxBranches];
     for (int b = 0; b < n_branches; ++b) {
-      const TD* x = (const TD*)a.x[b] + t * N;
+      const TD* xr = (const TD*)a.x[b] + t * N;
       float ss = 0.f;
-      for (int i = threadIdx.x; i < N; i += blockDim.x) {
-        const float v = to_f32<TD>(x[i]);
-        ss = fmaf(v, v, ss);
+      for (int i = threadIdx.x * V; i < N; i += step) {
+        get(xr + i, x);
+#pragma unroll
+        for (int k = 0; k < V; ++k) ss = fmaf(x[k], x[k], ss);
       }
       inv[b] = rsqrtf(block_sum(ss, red) / (float)N + eps);
     }
     const float share = 1.0f / (float)n_branches;
-    for (int i = threadIdx.x; i < N; i += blockDim.x) {
-      float y = 0.f;
-      for (int b = 0; b < n_branches; ++b) y += to_f32<TD>(((const TD*)a.x[b])[t * N + i]) * inv[b] * a.w[b][i];
-      yrow[i] = y * share;
+    for (int i = threadIdx.x * V; i < N; i += step) {
+#pragma unroll
+      for (int k = 0; k < V; ++k) y[k] = 0.f;
+      for (int b = 0; b < n_branches; ++b) {
+        get((const TD*)a.x[b] + t * N + i, x);
+        get(a.w[b] + i, w);
+#pragma unroll
+        for (int k = 0; k < V; ++k) y[k] += x[k] * inv[b] * w[k];
+      }
+#pragma unroll
+      for (int k = 0; k < V; ++k) y[k] *= share;
+      put(yrow + i, y);
     }
   }
   float ss = 0.f;
-  for (int i = threadIdx.x; i < N; i += blockDim.x) ss = fmaf(yrow[i], yrow[i], ss);   // (a thread reads what it wrote)
+  for (int i = threadIdx.x * V; i < N; i += step) {   // (a thread reads what it wrote)
+    get(yrow + i, y);
+#pragma unroll
+    for (int k = 0; k < V; ++k) ss = fmaf(y[k], y[k], ss);
+  }
   const float inv_y = rsqrtf(block_sum(ss, red) / (float)N + eps);
   float* hr = h + t * N;
   float s2 = 0.f;
-  for (int i = threadIdx.x; i < N; i += blockDim.x) {
-    const float v = hr[i] + yrow[i] * inv_y * w_post[i];
-    hr[i] = v;
-    yrow[i] = v;
-    s2 = fmaf(v, v, s2);
+  for (int i = threadIdx.x * V; i < N; i += step) {
+    get(yrow + i, y);
+    get(hr + i, x);
+    get(w_post + i, w);
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      x[k] += y[k] * inv_y * w[k];
+      s2 = fmaf(x[k], x[k], s2);
+    }
+    put(hr + i, x);
+    put(yrow + i, x);
   }
   if (!out) return;
   const float inv_h = rsqrtf(block_sum(s2, red) / (float)N + eps);
-  for (int i = threadIdx.x; i < N; i += blockDim.x) out[t * N + i] = from_f32<TO>(yrow[i] * inv_h * w_next[i]);
+  for (int i = threadIdx.x * V; i < N; i += step) {
+    get(yrow + i, x);
+    get(w_next + i, w);
+#pragma unroll
+    for (int k = 0; k < V; ++k) x[k] = x[k] * inv_h * w[k];
+    put(out + t * N + i, x);
+  }
 }
 
 // h float [T, N] in place; xs: n_branches tensors [T, N] of `d_dtype`, ws: their float weights [N] (ws[0] null with one
@@ -601,7 +640,13 @@ SHARPI_EXPORT int sharpi_post_pre_norm(float* h, const void* const* xs, const fl
     a.w[b] = ws[b];
   }
   const size_t lds = (size_t)N * sizeof(float);
-#define PPN(TD, TO) post_pre_norm_kernel<TD, TO><<<n_rows, 256, lds, stream>>>(h, a, n_branches, w_post, w_next, (TO*)out, N, eps)
+  bool wide = N % 8 == 0 && (uintptr_t)h % 32 == 0 && (uintptr_t)out % 32 == 0 && (uintptr_t)w_post % 32 == 0 && (uintptr_t)w_next % 32 == 0;
+  for (int b = 0; b < n_branches; ++b) wide = wide && (uintptr_t)xs[b] % 32 == 0 && (uintptr_t)ws[b] % 32 == 0;
+#define PPN(TD, TO)                                                                                                        \
+  do {                                                                                                                     \
+    if (wide) post_pre_norm_kernel<TD, TO, 8><<<n_rows, 256, lds, stream>>>(h, a, n_branches, w_post, w_next, (TO*)out, N, eps); \
+    else post_pre_norm_kernel<TD, TO, 1><<<n_rows, 256, lds, stream>>>(h, a, n_branches, w_post, w_next, (TO*)out, N, eps);      \
+  } while (0)
   const bool of = !out || o_dtype == DT_F32;
   if (out && o_dtype != DT_F32 && o_dtype != DT_BF16) return SHARPI_ERR_ARG;
   if (d_dtype == DT_F32) {

@@ -1,11 +1,15 @@
 // Gated linear attention: a matrix-valued recurrent state per head with a decay per key channel,
 //   S_t = diag(alpha_t) S_(t-1) + k_t v_t^T,   o_t = S_t^T q_t,   alpha_t = sigmoid(z_t)^(1/tau),
 // walked token by token in float.  The state of a request lives in its state slot and is carried
-// from step to step.  It is kept column slice by column slice, [slots, heads, ceil(dv / 8), dk, 8]
-// (float): the 8 columns a block owns are then one contiguous piece of memory, which the block
-// alone reads and writes (row-major [dk, dv], a block's 32 bytes of every row would share their
-// cache lines with three other blocks on other compute dies, and every line would cross the
-// memory interface four times).
+// from step to step.  It is kept column slice by column slice and, inside a slice, in the order the
+// walking wave's lanes hold it: [slots, heads, ceil(dv / 8), DKP, 8] floats with DKP the rows the
+// lanes cover (dk rounded up to 32, 64, 128 or 256), row g * RPL + r of the slice at place
+// r * 8 + g: the 8 columns a block owns are one contiguous piece of memory which the block alone
+// reads and writes, 256 bytes a load of the wave.
+//
+// Two forms: stages of 16 tokens (8 for the widest heads) for steps that bring portions of prompts,
+// and stages of 2 tokens for steps of single tokens, whose blocks then take 3 KB of LDS instead of
+// 50 and fill the chip (a decode step at batch 64 has 16,384 of them).
 //
 // A block owns kCols value columns of one head of one entry: the columns of S are independent of
 // each other, so an entry's work is spread over heads x ceil(dv / kCols) blocks, and the walk along
@@ -69,14 +73,14 @@ __global__ __launch_bounds__(256) void gla_decays_fused_kernel(const T* __restri
     if (tt < nt) alpha[(size_t)(t0 + tt) * N + c] = expf(log_sigmoid(acc[tt] + b) * inv_tau);
 }
 
-template <typename T, int RPL, bool VEC>
+template <typename T, int RPL, bool VEC, bool SHORT>
 __global__ __launch_bounds__(2 * kWave) void gla_walk_kernel(
     const T* __restrict__ proj, int stride, int q_off, int k_off, int v_off, const float* __restrict__ alpha,
     float q_scale, float* __restrict__ state,
     const int* __restrict__ state_slots, const int* __restrict__ cu_tokens, float* __restrict__ out, int nh, int dk,
     int dv) {
   constexpr int DKP = RPL * kGroups;               // rows the lanes cover; rows beyond dk stay zero
-  constexpr int kStage = DKP <= 128 ? 16 : 8;      // tokens staged at a time (two stages fit in LDS)
+  constexpr int kStage = SHORT ? 2 : DKP <= 128 ? 16 : 8;   // tokens staged at a time (two stages fit in LDS)
   __shared__ __attribute__((aligned(16))) float qs[2][kStage][DKP];
   __shared__ __attribute__((aligned(16))) float ks[2][kStage][DKP];
   __shared__ __attribute__((aligned(16))) float as[2][kStage][DKP];
@@ -88,13 +92,13 @@ __global__ __launch_bounds__(2 * kWave) void gla_walk_kernel(
   const int col = c0 + j;
   const bool col_ok = col < dv;
   const int first = cu_tokens[e], len = cu_tokens[e + 1] - first;
-  float* S = state + ((((size_t)state_slots[e] * nh + h) * gridDim.x + blockIdx.x) * dk) * kCols;
+  float* S = state + ((((size_t)state_slots[e] * nh + h) * gridDim.x + blockIdx.x) * DKP) * kCols;
   float s[RPL];
   if (walker) {
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
       const int rowi = g * RPL + r;
-      s[r] = (col_ok && rowi < dk) ? S[(size_t)rowi * kCols + j] : 0.f;
+      s[r] = (col_ok && rowi < dk) ? S[(r * kGroups + g) * kCols + j] : 0.f;
     }
   }
   auto stage = [&](int t0, int buf) {
@@ -197,7 +201,7 @@ __global__ __launch_bounds__(2 * kWave) void gla_walk_kernel(
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
       const int rowi = g * RPL + r;
-      if (col_ok && rowi < dk) S[(size_t)rowi * kCols + j] = s[r];
+      if (col_ok && rowi < dk) S[(r * kGroups + g) * kCols + j] = s[r];
     }
   }
 }
@@ -232,18 +236,23 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
 template <typename T>
 static int launch_walk(const void* proj, int stride, int q_off, int k_off, int v_off, const float* alpha, float q_scale,
                        float* state, const int* state_slots, const int* cu_tokens, float* out, int n_entries, int nh,
-                       int dk, int dv, hipStream_t stream) {
+                       int dk, int dv, int max_entry_len, hipStream_t stream) {
   dim3 grid(ceil_div(dv, kCols), nh, n_entries);
   const bool vec = dk % 8 == 0 && stride % 8 == 0 && q_off % 8 == 0 && k_off % 8 == 0 &&
                    ((uintptr_t)proj % 32 == 0) && ((uintptr_t)alpha % 32 == 0);
-#define WALK(RPL)                                                                                                    \
-  do {                                                                                                               \
-    if (vec)                                                                                                         \
-      gla_walk_kernel<T, RPL, true><<<grid, 2 * kWave, 0, stream>>>((const T*)proj, stride, q_off, k_off, v_off, alpha, \
-                                                                    q_scale, state, state_slots, cu_tokens, out, nh, dk, dv); \
-    else                                                                                                             \
-      gla_walk_kernel<T, RPL, false><<<grid, 2 * kWave, 0, stream>>>((const T*)proj, stride, q_off, k_off, v_off, alpha, \
-                                                                     q_scale, state, state_slots, cu_tokens, out, nh, dk, dv); \
+  const bool brief = max_entry_len <= 2;
+#define WALK_AS(RPL, VEC, SHORT)                                                                                      \
+  gla_walk_kernel<T, RPL, VEC, SHORT><<<grid, 2 * kWave, 0, stream>>>((const T*)proj, stride, q_off, k_off, v_off, alpha, \
+                                                                      q_scale, state, state_slots, cu_tokens, out, nh, dk, dv)
+#define WALK(RPL)                         \
+  do {                                    \
+    if (brief) {                          \
+      if (vec) WALK_AS(RPL, true, true);  \
+      else WALK_AS(RPL, false, true);     \
+    } else {                              \
+      if (vec) WALK_AS(RPL, true, false); \
+      else WALK_AS(RPL, false, false);    \
+    }                                     \
   } while (0)
   if (dk <= 32) WALK(4);
   else if (dk <= 64) WALK(8);
@@ -251,11 +260,11 @@ static int launch_walk(const void* proj, int stride, int q_off, int k_off, int v
   else if (dk <= 256) WALK(32);
   else return SHARPI_ERR_ARG;
 #undef WALK
+#undef WALK_AS
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
 }
 
-// z float [n_rows, N]: decay logits, turned in place into decays sigmoid(z + bias)^(1 / tau), bias [N].
 // columns of the state that lie together in memory (the state's layout is [.., ceil(dv / this), dk, this])
 SHARPI_EXPORT int sharpi_gla_state_cols() { return kCols; }
 
@@ -291,21 +300,22 @@ SHARPI_EXPORT int sharpi_gla_decays_fused(const void* proj, int dtype, int strid
 }
 
 // proj [T, stride] of `dtype` holds q (nh * dk columns at q_off), k (at k_off) and v (nh * dv at
-// v_off); alpha float [T, nh * dk] are the decays; state float [slots, nh, ceil(dv / 8), dk, 8]; out float
+// v_off); alpha float [T, nh * dk] are the decays; state float [slots, nh, ceil(dv / 8), DKP, 8] (see above);
+// max_entry_len bounds the tokens of an entry (it picks the form: stages of 2 tokens up to 2); out float
 // [T, nh * dv].  Entries (cu_tokens [entries + 1]) are walked in parallel, each from the state of
 // its slot, which is left advanced.
 SHARPI_EXPORT int sharpi_gla_walk(const void* proj, int dtype, int stride, int q_off, int k_off, int v_off,
                                   const float* alpha, float q_scale, float* state, const int* state_slots,
                                   const int* cu_tokens, float* out, int n_entries, int nh, int dk, int dv,
-                                  hipStream_t stream) {
+                                  int max_entry_len, hipStream_t stream) {
   if (n_entries <= 0) return SHARPI_OK;
   if (nh <= 0 || nh > 65535 || n_entries > 65535 || dk <= 0 || dk > 256 || dv <= 0) return SHARPI_ERR_ARG;
   if (dtype == DT_F32)
     return launch_walk<float>(proj, stride, q_off, k_off, v_off, alpha, q_scale, state, state_slots, cu_tokens, out,
-                              n_entries, nh, dk, dv, stream);
+                              n_entries, nh, dk, dv, max_entry_len, stream);
   if (dtype == DT_BF16)
     return launch_walk<bf16_t>(proj, stride, q_off, k_off, v_off, alpha, q_scale, state, state_slots, cu_tokens, out,
-                               n_entries, nh, dk, dv, stream);
+                               n_entries, nh, dk, dv, max_entry_len, stream);
   return SHARPI_ERR_ARG;
 }
 

@@ -1187,17 +1187,26 @@ GLA_MAX_KEY_DIM = 256      # key channels of a head that the walk holds (csrc/li
 GLA_STATE_COLS = _lib.GLA_STATE_COLS   # value columns of the state that lie together in memory (checked against the library at load)
 
 
+def _gla_rows(dk: int) -> int:
+    """Rows of a state slice as the walk's lanes cover them: dk rounded up to 32, 64, 128 or 256."""
+    return 32 if dk <= 32 else 64 if dk <= 64 else 128 if dk <= 128 else 256
+
+
 def gla_state_shape(nh: int, dk: int, dv: int) -> tuple:
-    """A request's recurrent state as the walk keeps it: [heads, ceil(dv / 8), dk, 8], column slice by
-    column slice (element (h, i, j) of the matrices S_h [dk, dv] lies at [h, j // 8, i, j % 8])."""
-    return (nh, (dv + GLA_STATE_COLS - 1) // GLA_STATE_COLS, dk, GLA_STATE_COLS)
+    """A request's recurrent state as the walk keeps it: [heads, ceil(dv / 8), DKP, 8], column slice by
+    column slice, DKP = dk rounded up to 32 / 64 / 128 / 256; inside a slice row i = g * (DKP / 8) + r
+    lies at place r * 8 + g (the order the walking wave's lanes hold it in)."""
+    return (nh, (dv + GLA_STATE_COLS - 1) // GLA_STATE_COLS, _gla_rows(dk), GLA_STATE_COLS)
 
 
-def gla_state_matrices(state: torch.Tensor, dv: int) -> torch.Tensor:
-    """[.., heads, ceil(dv / 8), dk, 8] as kept -> the matrices [.., heads, dk, dv] (a copy; for tests and tools)."""
-    *lead, nh, ncb, dk, c = state.shape
-    return state.movedim(-3, -2).reshape(*lead, nh, dk, ncb * c)[..., :dv].contiguous()
-
+def gla_state_matrices(state: torch.Tensor, dk: int, dv: int) -> torch.Tensor:
+    """The state as kept -> the matrices [.., heads, dk, dv] (a copy; for tests and tools)."""
+    *lead, nh, ncb, dkp, c = state.shape
+    rpl = dkp // 8
+    m = state.reshape(*lead, nh, ncb, rpl, 8, c)                 # [.., h, slice, r, g, j]
+    m = m.movedim(-2, -3)                                        # [.., h, slice, g, r, j]: row g * rpl + r
+    m = m.reshape(*lead, nh, ncb, dkp, c).movedim(-3, -2)        # [.., h, row, slice, j]
+    return m.reshape(*lead, nh, dkp, ncb * c)[..., :dk, :dv].contiguous()
 
 
 def gla_decays(z: torch.Tensor, bias: torch.Tensor, tau: float) -> torch.Tensor:
@@ -1243,13 +1252,13 @@ def gla_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, alpha: torc
           "gla_walk: q, k and v columns must lie inside proj")
     _need(alpha.dtype == torch.float32 and alpha.shape == (T, nh * dk), "gla_walk: alpha float32 [T, nh*dk] wanted")
     _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == gla_state_shape(nh, dk, dv),
-          "gla_walk: state must be float32 [slots, nh, ceil(dv / 8), dk, 8]")
+          "gla_walk: state must be float32 [slots, *gla_state_shape(nh, dk, dv)]")
     _need(ctx.state_slots.shape == (ctx.n_entries,) and ctx.cu_tokens.shape == (ctx.n_entries + 1,) and ctx.n_tokens == T,
           "gla_walk: the step's per-entry arrays do not fit")
     out = torch.empty(T, nh * dv, dtype=torch.float32, device=proj.device)
     _run("sharpi_gla_walk", _ptr(proj), _code(proj.dtype), N, int(q_off), int(k_off), int(v_off), _ptr(alpha),
          float(q_scale), _ptr(state), _ptr(ctx.state_slots), _ptr(ctx.cu_tokens), _ptr(out), ctx.n_entries,
-         nh, dk, dv, _stream())
+         nh, dk, dv, int(getattr(ctx, "max_entry_len", 0) or T), _stream())
     return out
 
 

@@ -49,7 +49,7 @@ class _Step:
     """What the kernels between projections and attention read of a step."""
 
     def __init__(self, lens, starts, slots):
-        self.n_entries, self.n_tokens = len(lens), sum(lens)
+        self.n_entries, self.n_tokens, self.max_entry_len = len(lens), sum(lens), max(lens)
         cu = [0]
         for n in lens:
             cu.append(cu[-1] + n)
@@ -152,15 +152,16 @@ def test_convolution_norm_rotation_and_cache_write(dtype, H, G, d, e, norm, layo
 @pytest.mark.parametrize("H, dk, dv, tau", [(2, 10, 24, 3.0), (6, 48, 64, 16.0), (1, 136, 20, 0.5), (3, 72, 50, 1.0), (2, 256, 16, 4.0),
                                             (4, 32, 33, 8.0)])
 def test_the_recurrence_walks_every_entry_from_its_slots_state(dtype, H, dk, dv, tau):
-    """Three requests over three steps (one token, a few, many; a request left out of a step) against
+    """Three requests over five steps (one token, a few, many; a request left out of a step) against
     the plain recurrence over whole sequences; states in slots 3, 0 and 1 of five."""
     from sharpinference_amd import ops
 
     g = torch.Generator().manual_seed(dk + dv)
     qk, vv = H * dk, H * dv
     pad = 3 if dk % 16 else 8                                    # (rows of eight aligned elements take the wide loads)
-    plan = [[("a", 1), ("b", 40)], [("b", 1), ("c", 7), ("a", 2)], [("a", 9), ("c", 1)]]
-    total = {"a": 12, "b": 41, "c": 8}
+    plan = [[("a", 1), ("b", 40)], [("b", 1), ("c", 7), ("a", 2)], [("a", 9), ("c", 1)],
+            [("c", 1), ("a", 2), ("b", 1)], [("b", 1)]]           # (the last two: single tokens and pairs only, the short-stage form)
+    total = {"a": 14, "b": 43, "c": 9}
     slot_of = {"a": 3, "b": 0, "c": 1}
     proj = {r: torch.randn(n, pad + 2 * qk + vv, generator=g).to(DT[dtype]) for r, n in total.items()}
     z = {r: torch.randn(n, qk, generator=g) * 2 for r, n in total.items()}
@@ -196,7 +197,7 @@ def test_the_recurrence_walks_every_entry_from_its_slots_state(dtype, H, dk, dv,
         S = torch.zeros(H, dk, dv, dtype=torch.float64)
         for t in range(n):
             S = alpha[t][:, :, None] * S + k[t][:, :, None] * v[t][:, None, :]
-        got_S = ops.gla_state_matrices(state[slot_of[r]], dv).cpu()
+        got_S = ops.gla_state_matrices(state[slot_of[r]], dk, dv).cpu()
         assert _rel_rms(got_S.reshape(1, -1), S.reshape(1, -1)) < 2e-6, f"state of {r}"
 
 
