@@ -7,16 +7,29 @@
 // r * 8 + g: the 8 columns a block owns are one contiguous piece of memory which the block alone
 // reads and writes, 256 bytes a load of the wave.
 //
-// Two forms: stages of 16 tokens (8 for the widest heads) for steps that bring portions of prompts,
-// and stages of 2 tokens for steps of single tokens, whose blocks then take 3 KB of LDS instead of
-// 50 and fill the chip (a decode step at batch 64 has 16,384 of them).
+// A long entry (a prompt alone in its step leaves most of the chip idle: 256 blocks for 16 heads of 128
+// value columns) can be walked in segments: phase 1 walks every segment but an entry's last from a
+// zero state and leaves its local state and the product D of its decays; a short kernel then turns the
+// local states into the segments' true start states, S_start(n + 1) = D_n S_start(n) + S_local(n), one
+// after the other from the slot's state; phase 2 walks every segment again from its start state, now
+// writing outputs, and the last segment leaves the entry's new state in the slot.  Twice the sums
+// on as many times the blocks as an entry has segments; the results differ from the unsegmented
+// walk's by rounding only (the state at a segment's start is summed in another order).
 //
-// A block owns kCols value columns of one head of one entry: the columns of S are independent of
-// each other, so an entry's work is spread over heads x ceil(dv / kCols) blocks, and the walk along
-// the entry's tokens is the only thing that is sequential.  The block is two waves.  One walks:
+// Three forms: stages of 16 tokens (8 for the widest heads) for whole entries of steps that bring
+// portions of prompts; stages of 8 tokens for the segmented walk, whose many blocks then sit six to a
+// compute unit instead of three; and stages of 2 tokens for steps of single tokens, whose blocks take
+// 3 KB of LDS instead of 50 and fill the chip (a decode step at batch 64 has 16,384 of them).
+//
+// The columns of S are independent of each other, so an entry's work is spread over heads x
+// ceil(dv / 16) blocks, and the walk along
+// the entry's tokens is the only thing that is sequential.  A block is two waves and takes kCPL
+// adjacent slices of kCols columns (a lane holds its rows of one column of each: every q, k and decay
+// read from LDS then feeds two columns' sums; with one column a lane the walk was bound by LDS reads).
+// The walking wave:
 // lane (g, j) holds RPL consecutive rows of column j (rows g * RPL ...); per token it scales its rows
 // by alpha, adds k[row] * v[j], and sums S[row][j] * q[row] over its rows; the row groups are then
-// added by exchanges between lanes.  The other wave runs a stage ahead: it fetches q, k, v and the
+// added by exchanges between lanes.  The staging wave runs a stage ahead: it fetches q, k, v and the
 // decays of the next kStage tokens (16 bytes a load where sizes and offsets are multiples of
 // eight) and leaves them in the other half of LDS, so that the walking wave reads LDS only and
 // never waits for memory.  Every sum's order depends on (dk, dv) alone: a token's output has the
@@ -26,8 +39,9 @@
 // float: alpha = exp(log_sigmoid(z + bias) / tau), in place over the logits.
 #include "common.h"
 
-constexpr int kCols = 8;                 // value columns a block owns
+constexpr int kCols = 8;                 // value columns a walking wave owns
 constexpr int kGroups = kWave / kCols;   // row groups
+constexpr int kCPL = 2;                  // columns a lane holds: a wave walks kCPL adjacent slices of kCols columns
 
 // log(sigmoid(z)) without overflow: min(z, 0) - log1p(exp(-|z|))
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
@@ -73,32 +87,55 @@ __global__ __launch_bounds__(256) void gla_decays_fused_kernel(const T* __restri
     if (tt < nt) alpha[(size_t)(t0 + tt) * N + c] = expf(log_sigmoid(acc[tt] + b) * inv_tau);
 }
 
-template <typename T, int RPL, bool VEC, bool SHORT>
+template <typename T, int RPL, bool VEC, int STAGE>
 __global__ __launch_bounds__(2 * kWave) void gla_walk_kernel(
     const T* __restrict__ proj, int stride, int q_off, int k_off, int v_off, const float* __restrict__ alpha,
     float q_scale, float* __restrict__ state,
     const int* __restrict__ state_slots, const int* __restrict__ cu_tokens, float* __restrict__ out, int nh, int dk,
-    int dv) {
+    int dv, int ncb, const int* __restrict__ segs, int phase, float* __restrict__ seg_state, float* __restrict__ seg_decay) {
   constexpr int DKP = RPL * kGroups;               // rows the lanes cover; rows beyond dk stay zero
-  constexpr int kStage = SHORT ? 2 : DKP <= 128 ? 16 : 8;   // tokens staged at a time (two stages fit in LDS)
+  constexpr int kStage = (STAGE > 8 && DKP > 128) ? 8 : STAGE;   // tokens staged at a time (two stages fit in LDS)
   __shared__ __attribute__((aligned(16))) float qs[2][kStage][DKP];
   __shared__ __attribute__((aligned(16))) float ks[2][kStage][DKP];
   __shared__ __attribute__((aligned(16))) float as[2][kStage][DKP];
-  __shared__ float vs[2][kStage][kCols];
-  const int e = blockIdx.z, h = blockIdx.y, c0 = blockIdx.x * kCols;
+  __shared__ float vs[2][kStage][kCPL * kCols];
+  __shared__ float part[kStage][kGroups][kCPL * kCols];   // the row groups' shares of a stage's outputs
+  // whole entries (segs null, phase 0): blockIdx.z is an entry.  Segments: blockIdx.z is a segment
+  // (entry, first token, tokens, 1 if the entry's last); phase 1 walks from zero and keeps the local
+  // state and the decays' product, phase 2 walks from the segment's start state and writes outputs.
+  int e = blockIdx.z, seg_first = 0, seg_len = 0;
+  bool seg_last = true;
+  if (segs) {
+    e = segs[4 * blockIdx.z];
+    seg_first = segs[4 * blockIdx.z + 1];
+    seg_len = segs[4 * blockIdx.z + 2];
+    seg_last = segs[4 * blockIdx.z + 3] != 0;
+    if (phase == 1 && seg_last) return;             // (nobody reads the local state of an entry's last segment)
+  }
+  const int h = blockIdx.y;
+  const int slice = blockIdx.x * kCPL;              // the first of the block's 8-column slices of the state
+  const int c0 = slice * kCols;
   const int lane = threadIdx.x & (kWave - 1);
   const bool walker = threadIdx.x < kWave;
-  const int j = lane % kCols, g = lane / kCols;
-  const int col = c0 + j;
-  const bool col_ok = col < dv;
-  const int first = cu_tokens[e], len = cu_tokens[e + 1] - first;
-  float* S = state + ((((size_t)state_slots[e] * nh + h) * gridDim.x + blockIdx.x) * DKP) * kCols;
-  float s[RPL];
+  const int j = lane % kCols, g = lane / kCols;     // the lane's columns: c0 + j and c0 + kCols + j; its rows: g * RPL ...
+  const int first = segs ? seg_first : cu_tokens[e], len = segs ? seg_len : cu_tokens[e + 1] - first;
+  float* S_slot = state + ((((size_t)state_slots[e] * nh + h) * ncb + slice) * DKP) * kCols;
+  float* S_seg = segs ? seg_state + ((((size_t)blockIdx.z * nh + h) * ncb + slice) * DKP) * kCols : nullptr;
+  const float* S_in = phase == 0 ? S_slot : phase == 2 ? S_seg : nullptr;
+  float* S = phase == 0 ? S_slot : phase == 1 ? S_seg : (seg_last ? S_slot : nullptr);    // where the state is left
+  const bool track = phase == 1;
+  float s[kCPL][RPL], dprod[RPL];
+  bool col_ok[kCPL];
+#pragma unroll
+  for (int c = 0; c < kCPL; ++c) col_ok[c] = c0 + c * kCols + j < dv;
   if (walker) {
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
       const int rowi = g * RPL + r;
-      s[r] = (col_ok && rowi < dk) ? S[(r * kGroups + g) * kCols + j] : 0.f;
+#pragma unroll
+      for (int c = 0; c < kCPL; ++c)      // (slice c of the block lies DKP * kCols floats behind slice c - 1)
+        s[c][r] = (S_in && col_ok[c] && rowi < dk) ? S_in[(size_t)c * DKP * kCols + (r * kGroups + g) * kCols + j] : 0.f;
+      dprod[r] = 1.f;
     }
   }
   auto stage = [&](int t0, int buf) {
@@ -148,9 +185,25 @@ __global__ __launch_bounds__(2 * kWave) void gla_walk_kernel(
         as[buf][tt][d] = av;
       }
     }
-    for (int i = lane; i < nt * kCols; i += kWave) {
-      const int tt = i / kCols, c = c0 + i % kCols;
-      vs[buf][tt][i % kCols] = c < dv ? to_f32<T>(proj[(size_t)(first + t0 + tt) * stride + v_off + h * dv + c]) : 0.f;
+    constexpr int VC = kCPL * kCols;                                 // the block's value columns
+    for (int i = lane; i < nt * VC; i += kWave) {
+      const int tt = i / VC, c = blockIdx.x * VC + i % VC;
+      vs[buf][tt][i % VC] = c < dv ? to_f32<T>(proj[(size_t)(first + t0 + tt) * stride + v_off + h * dv + c]) : 0.f;
+    }
+  };
+  // The outputs of a stage: its tokens' sums over the eight row groups, added in the order of the groups
+  // and written 64 bytes a token.  The walking wave does it at the start of the next stage (a barrier lies
+  // between; its own reads of `part` come before its next writes in program order), so that no exchange
+  // between lanes stands between one token's sums and the next one's.
+  int done_t0 = -1, done_nt = 0;
+  auto flush = [&]() {
+    constexpr int VC = kCPL * kCols;
+    for (int i = lane; i < done_nt * VC; i += kWave) {
+      const int tt = i / VC, c = i % VC;
+      float o = 0.f;
+#pragma unroll
+      for (int gg = 0; gg < kGroups; ++gg) o += part[tt][gg][c];
+      if (c0 + c < dv) out[(size_t)(first + done_t0 + tt) * (size_t)(nh * dv) + h * dv + c0 + c] = o;
     }
   };
   if (!walker) stage(0, 0);
@@ -161,8 +214,11 @@ __global__ __launch_bounds__(2 * kWave) void gla_walk_kernel(
       if (t0 + kStage < len) stage(t0 + kStage, buf ^ 1);
     } else {
       const int nt = min(kStage, len - t0);
+      if (!track && done_t0 >= 0) flush();
+      done_t0 = t0;
+      done_nt = nt;
       auto one_token = [&](int tt) {
-        const float v = vs[buf][tt][j];
+        const float v0 = vs[buf][tt][j], v1 = vs[buf][tt][kCols + j];
         const float* qrow = &qs[buf][tt][g * RPL];
         const float* krow = &ks[buf][tt][g * RPL];
         const float* arow = &as[buf][tt][g * RPL];
@@ -172,20 +228,19 @@ __global__ __launch_bounds__(2 * kWave) void gla_walk_kernel(
           const float4 a4 = *reinterpret_cast<const float4*>(arow + r);
           const float4 k4 = *reinterpret_cast<const float4*>(krow + r);
           const float4 q4 = *reinterpret_cast<const float4*>(qrow + r);
-          s[r + 0] = fmaf(a4.x, s[r + 0], k4.x * v);
-          o0 = fmaf(s[r + 0], q4.x, o0);
-          s[r + 1] = fmaf(a4.y, s[r + 1], k4.y * v);
-          o1 = fmaf(s[r + 1], q4.y, o1);
-          s[r + 2] = fmaf(a4.z, s[r + 2], k4.z * v);
-          o0 = fmaf(s[r + 2], q4.z, o0);
-          s[r + 3] = fmaf(a4.w, s[r + 3], k4.w * v);
-          o1 = fmaf(s[r + 3], q4.w, o1);
+          const float av[4] = {a4.x, a4.y, a4.z, a4.w}, kv[4] = {k4.x, k4.y, k4.z, k4.w}, qv[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+          for (int x = 0; x < 4; ++x) {
+            s[0][r + x] = fmaf(av[x], s[0][r + x], kv[x] * v0);
+            o0 = fmaf(s[0][r + x], qv[x], o0);
+            s[1][r + x] = fmaf(av[x], s[1][r + x], kv[x] * v1);
+            o1 = fmaf(s[1][r + x], qv[x], o1);
+            if (track) dprod[r + x] *= av[x];
+          }
         }
-        float o = o0 + o1;
-        o += __shfl_xor(o, 8, kWave);
-        o += __shfl_xor(o, 16, kWave);
-        o += __shfl_xor(o, 32, kWave);
-        if (g == 0 && col_ok) out[(size_t)(first + t0 + tt) * (size_t)(nh * dv) + h * dv + col] = o;
+        if (track) return;                            // (phase 1 wants the state and the decays only)
+        part[tt][g][j] = o0;                          // the groups' shares meet in `flush`, a stage later
+        part[tt][g][kCols + j] = o1;
       };
       if (nt == kStage) {
         // a full stage, unrolled: the LDS reads of the tokens ahead are requested while this one is summed
@@ -197,11 +252,63 @@ __global__ __launch_bounds__(2 * kWave) void gla_walk_kernel(
     }
     __syncthreads();
   }
-  if (walker) {
+  if (walker && !track && done_t0 >= 0) flush();     // (the loop's last barrier lies before this)
+  if (walker && S) {
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
       const int rowi = g * RPL + r;
-      if (col_ok && rowi < dk) S[(r * kGroups + g) * kCols + j] = s[r];
+#pragma unroll
+      for (int c = 0; c < kCPL; ++c)
+        if (col_ok[c] && rowi < dk) S[(size_t)c * DKP * kCols + (r * kGroups + g) * kCols + j] = s[c][r];
+    }
+  }
+  if (walker && track && slice == 0 && j == 0) {
+#pragma unroll
+    for (int r = 0; r < RPL; ++r) seg_decay[((size_t)blockIdx.z * nh + h) * DKP + g * RPL + r] = dprod[r];
+  }
+}
+
+// Between the two phases of a segmented walk: an entry's segments one after the other.  The state at the
+// first segment's start is the slot's; S_start(n + 1) = D_n S_start(n) + S_local(n).  seg_state holds
+// S_local on entry and S_start on exit.  One wave a (column slice, head, entry), lanes as in the walk.
+template <int RPL>
+__global__ __launch_bounds__(kWave) void gla_combine_kernel(const float* __restrict__ state, const int* __restrict__ state_slots,
+                                                            const int* __restrict__ ent_segs, float* __restrict__ seg_state,
+                                                            const float* __restrict__ seg_decay, int nh) {
+  constexpr int DKP = RPL * kGroups;
+  const int e = blockIdx.z, h = blockIdx.y;
+  const int lane = threadIdx.x, j = lane % kCols, g = lane / kCols;
+  const int seg0 = ent_segs[2 * e], n = ent_segs[2 * e + 1];
+  const float* S_slot = state + ((((size_t)state_slots[e] * nh + h) * gridDim.x + blockIdx.x) * DKP) * kCols;
+  float s[RPL];
+#pragma unroll
+  for (int r = 0; r < RPL; ++r) s[r] = S_slot[(r * kGroups + g) * kCols + j];
+  // (a segment's local state and decays are requested one segment ahead of their use: the chain of
+  // sums is short, the loads are what takes time)
+  float local[RPL] = {}, dec[RPL] = {};
+  auto fetch = [&](int i) {
+    const size_t seg = (size_t)(seg0 + i);
+    const float* p = seg_state + (((seg * nh + h) * gridDim.x + blockIdx.x) * DKP) * kCols;
+    const float* d = seg_decay + (seg * nh + h) * DKP + g * RPL;
+#pragma unroll
+    for (int r = 0; r < RPL; ++r) {
+      local[r] = p[(r * kGroups + g) * kCols + j];
+      dec[r] = d[r];
+    }
+  };
+  if (n > 1) fetch(0);
+  for (int i = 0; i < n; ++i) {
+    float* p = seg_state + ((((size_t)(seg0 + i) * nh + h) * gridDim.x + blockIdx.x) * DKP) * kCols;
+    float next[RPL];
+#pragma unroll
+    for (int r = 0; r < RPL; ++r) {
+      p[(r * kGroups + g) * kCols + j] = s[r];
+      next[r] = fmaf(dec[r], s[r], local[r]);
+    }
+    if (i + 2 < n) fetch(i + 1);                       // (the last segment has no local state to read)
+    if (i + 1 < n) {
+#pragma unroll
+      for (int r = 0; r < RPL; ++r) s[r] = next[r];
     }
   }
 }
@@ -237,21 +344,23 @@ template <typename T>
 static int launch_walk(const void* proj, int stride, int q_off, int k_off, int v_off, const float* alpha, float q_scale,
                        float* state, const int* state_slots, const int* cu_tokens, float* out, int n_entries, int nh,
                        int dk, int dv, int max_entry_len, hipStream_t stream) {
-  dim3 grid(ceil_div(dv, kCols), nh, n_entries);
+  const int ncb = ceil_div(dv, kCols);
+  dim3 grid(ceil_div(ncb, kCPL), nh, n_entries);
   const bool vec = dk % 8 == 0 && stride % 8 == 0 && q_off % 8 == 0 && k_off % 8 == 0 &&
                    ((uintptr_t)proj % 32 == 0) && ((uintptr_t)alpha % 32 == 0);
   const bool brief = max_entry_len <= 2;
-#define WALK_AS(RPL, VEC, SHORT)                                                                                      \
-  gla_walk_kernel<T, RPL, VEC, SHORT><<<grid, 2 * kWave, 0, stream>>>((const T*)proj, stride, q_off, k_off, v_off, alpha, \
-                                                                      q_scale, state, state_slots, cu_tokens, out, nh, dk, dv)
+#define WALK_AS(RPL, VEC, STAGE)                                                                                      \
+  gla_walk_kernel<T, RPL, VEC, STAGE><<<grid, 2 * kWave, 0, stream>>>(                                       \
+      (const T*)proj, stride, q_off, k_off, v_off, alpha, q_scale, state, state_slots, cu_tokens, out, nh, dk, dv, ncb, nullptr, 0, \
+      nullptr, nullptr)
 #define WALK(RPL)                         \
   do {                                    \
     if (brief) {                          \
-      if (vec) WALK_AS(RPL, true, true);  \
-      else WALK_AS(RPL, false, true);     \
+      if (vec) WALK_AS(RPL, true, 2);     \
+      else WALK_AS(RPL, false, 2);        \
     } else {                              \
-      if (vec) WALK_AS(RPL, true, false); \
-      else WALK_AS(RPL, false, false);    \
+      if (vec) WALK_AS(RPL, true, 16);    \
+      else WALK_AS(RPL, false, 16);       \
     }                                     \
   } while (0)
   if (dk <= 32) WALK(4);
@@ -263,6 +372,59 @@ static int launch_walk(const void* proj, int stride, int q_off, int k_off, int v
 #undef WALK_AS
   SHARPI_CHECK_LAUNCH();
   return SHARPI_OK;
+}
+
+template <typename T>
+static int launch_segmented(const void* proj, int stride, int q_off, int k_off, int v_off, const float* alpha, float q_scale,
+                            float* state, const int* state_slots, const int* cu_tokens, float* out, int n_entries, int nh,
+                            int dk, int dv, const int* segs, const int* ent_segs, int n_segs, float* seg_state,
+                            float* seg_decay, hipStream_t stream) {
+  const int ncb = ceil_div(dv, kCols);
+  dim3 grid(ceil_div(ncb, kCPL), nh, n_segs), cgrid(ncb, nh, n_entries);
+  const bool vec = dk % 8 == 0 && stride % 8 == 0 && q_off % 8 == 0 && k_off % 8 == 0 &&
+                   ((uintptr_t)proj % 32 == 0) && ((uintptr_t)alpha % 32 == 0);
+#define PHASE(RPL, VEC, PH)                                                                                            \
+  gla_walk_kernel<T, RPL, VEC, 8><<<grid, 2 * kWave, 0, stream>>>(                                         \
+      (const T*)proj, stride, q_off, k_off, v_off, alpha, q_scale, state, state_slots, cu_tokens, out, nh, dk, dv, ncb, segs, PH, \
+      seg_state, seg_decay)
+#define SEGMENTED(RPL)                                                                                       \
+  do {                                                                                                       \
+    if (vec) PHASE(RPL, true, 1);                                                                            \
+    else PHASE(RPL, false, 1);                                                                               \
+    gla_combine_kernel<RPL><<<cgrid, kWave, 0, stream>>>(state, state_slots, ent_segs, seg_state, seg_decay, nh); \
+    if (vec) PHASE(RPL, true, 2);                                                                            \
+    else PHASE(RPL, false, 2);                                                                               \
+  } while (0)
+  if (dk <= 32) SEGMENTED(4);
+  else if (dk <= 64) SEGMENTED(8);
+  else if (dk <= 128) SEGMENTED(16);
+  else if (dk <= 256) SEGMENTED(32);
+  else return SHARPI_ERR_ARG;
+#undef SEGMENTED
+#undef PHASE
+  SHARPI_CHECK_LAUNCH();
+  return SHARPI_OK;
+}
+
+// The walk of gla_walk with long entries cut into segments that are walked side by side (see the head of
+// this file).  segs int [n_segs, 4] = (entry, first token of the step's rows, tokens, 1 if the entry's last
+// segment), an entry's segments consecutive and in order; ent_segs int [n_entries, 2] = (first segment,
+// segments); seg_state float [n_segs, nh, ceil(dv / 8), DKP, 8] and seg_decay float [n_segs, nh, DKP]: scratch.
+SHARPI_EXPORT int sharpi_gla_walk_segmented(const void* proj, int dtype, int stride, int q_off, int k_off, int v_off,
+                                            const float* alpha, float q_scale, float* state, const int* state_slots,
+                                            const int* cu_tokens, float* out, int n_entries, int nh, int dk, int dv,
+                                            const int* segs, const int* ent_segs, int n_segs, float* seg_state,
+                                            float* seg_decay, hipStream_t stream) {
+  if (n_entries <= 0 || n_segs <= 0) return SHARPI_OK;
+  if (nh <= 0 || nh > 65535 || n_entries > 65535 || n_segs > 65535 || dk <= 0 || dk > 256 || dv <= 0) return SHARPI_ERR_ARG;
+  if (!segs || !ent_segs || !seg_state || !seg_decay) return SHARPI_ERR_ARG;
+  if (dtype == DT_F32)
+    return launch_segmented<float>(proj, stride, q_off, k_off, v_off, alpha, q_scale, state, state_slots, cu_tokens, out,
+                                   n_entries, nh, dk, dv, segs, ent_segs, n_segs, seg_state, seg_decay, stream);
+  if (dtype == DT_BF16)
+    return launch_segmented<bf16_t>(proj, stride, q_off, k_off, v_off, alpha, q_scale, state, state_slots, cu_tokens, out,
+                                    n_entries, nh, dk, dv, segs, ent_segs, n_segs, seg_state, seg_decay, stream);
+  return SHARPI_ERR_ARG;
 }
 
 // columns of the state that lie together in memory (the state's layout is [.., ceil(dv / this), dk, this])

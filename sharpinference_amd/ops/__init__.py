@@ -1239,12 +1239,33 @@ def gla_decays_from_middle(proj: torch.Tensor, a_off: int, rank: int, w: torch.T
     return alpha
 
 
+GLA_SEGMENT_TOKENS = 128       # tokens of a segment of the segmented walk
+
+
+def gla_segments(lens, cu_tokens):
+    """The work lists of the segmented walk for entries of `lens` tokens whose rows start at
+    `cu_tokens`: (segs int32 [n, 4] = (entry, first row, tokens, 1 if the entry's last), ent_segs int32
+    [entries, 2] = (first segment, segments)), as numpy arrays."""
+    import numpy as np
+
+    segs, ents = [], []
+    for e, n in enumerate(lens):
+        first = len(segs)
+        for o in range(0, n, GLA_SEGMENT_TOKENS):
+            m = min(GLA_SEGMENT_TOKENS, n - o)
+            segs.append((e, int(cu_tokens[e]) + o, m, 1 if o + m == n else 0))
+        ents.append((first, len(segs) - first))
+    return np.asarray(segs, dtype=np.int32).reshape(-1, 4), np.asarray(ents, dtype=np.int32).reshape(-1, 2)
+
+
 def gla_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, alpha: torch.Tensor, q_scale: float,
-             state: torch.Tensor, ctx, nh: int, dk: int, dv: int) -> torch.Tensor:
+             state: torch.Tensor, ctx, nh: int, dk: int, dv: int, segments=None) -> torch.Tensor:
     """The recurrence S_t = diag(alpha_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per head, token by
     token along every entry of the step, from and into state [slots, *gla_state_shape(nh, dk, dv)]
     (float32) at the entries' state slots.  q, k (nh*dk columns each) and v (nh*dv) are columns of proj [T, N]; q is
-    multiplied by q_scale; alpha float32 [T, nh*dk] are the decays.  Returns o float32 [T, nh*dv]."""
+    multiplied by q_scale; alpha float32 [T, nh*dk] are the decays.  Returns o float32 [T, nh*dv].
+    ``segments`` = (segs, ent_segs) on the device (see :func:`gla_segments`): long entries are then walked
+    segment by segment side by side (results equal to rounding)."""
     _dev(proj, alpha, state)
     T, N = proj.shape
     _need(1 <= dk <= GLA_MAX_KEY_DIM and dv >= 1 and nh >= 1, f"gla_walk: key channels 1..{GLA_MAX_KEY_DIM}")
@@ -1256,6 +1277,20 @@ def gla_walk(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, alpha: torc
     _need(ctx.state_slots.shape == (ctx.n_entries,) and ctx.cu_tokens.shape == (ctx.n_entries + 1,) and ctx.n_tokens == T,
           "gla_walk: the step's per-entry arrays do not fit")
     out = torch.empty(T, nh * dv, dtype=torch.float32, device=proj.device)
+    if segments is not None:
+        segs, ent_segs = segments
+        _dev(segs, ent_segs)
+        _i32(segs, "segs")
+        _i32(ent_segs, "ent_segs")
+        n_segs = segs.numel() // 4
+        _need(segs.numel() == 4 * n_segs and ent_segs.numel() == 2 * ctx.n_entries and n_segs >= ctx.n_entries,
+              "gla_walk: segs [n, 4] and ent_segs [entries, 2] wanted")
+        seg_state = torch.empty((n_segs,) + gla_state_shape(nh, dk, dv), dtype=torch.float32, device=proj.device)
+        seg_decay = torch.empty(n_segs, nh, _gla_rows(dk), dtype=torch.float32, device=proj.device)
+        _run("sharpi_gla_walk_segmented", _ptr(proj), _code(proj.dtype), N, int(q_off), int(k_off), int(v_off), _ptr(alpha),
+             float(q_scale), _ptr(state), _ptr(ctx.state_slots), _ptr(ctx.cu_tokens), _ptr(out), ctx.n_entries, nh, dk, dv,
+             _ptr(segs), _ptr(ent_segs), n_segs, _ptr(seg_state), _ptr(seg_decay), _stream())
+        return out
     _run("sharpi_gla_walk", _ptr(proj), _code(proj.dtype), N, int(q_off), int(k_off), int(v_off), _ptr(alpha),
          float(q_scale), _ptr(state), _ptr(ctx.state_slots), _ptr(ctx.cu_tokens), _ptr(out), ctx.n_entries,
          nh, dk, dv, int(getattr(ctx, "max_entry_len", 0) or T), _stream())

@@ -52,6 +52,7 @@ _SIGNATURES = {
     "sharpi_qk_prep": [P, I, I, I, I, I, I, I, I, I, I, I, P, I, P, P, P, P, P, I, P, P, F, P, I, I, F, P, P, P, P, I, I, P],
     "sharpi_gla_walk": [P, I, I, I, I, I, P, F, P, P, P, P, I, I, I, I, I, P],
     "sharpi_gla_decays": [P, P, F, I, I, P],
+    "sharpi_gla_walk_segmented": [P, I, I, I, I, I, P, F, P, P, P, P, I, I, I, I, P, P, I, P, P, P],
     "sharpi_gla_decays_fused": [P, I, I, I, I, P, P, F, P, I, I, P],
     "sharpi_head_norm_gate": [P, P, F, P, I, I, I, P, I, I, I, P],
     "sharpi_activation": [P, P, I, c_longlong, I, P],

@@ -1,14 +1,38 @@
 """The gated linear attention mixer: a matrix-valued state per head instead of a cache of keys."""
 from __future__ import annotations
 
-from typing import Dict, Optional
+from typing import Dict, List, Optional, Tuple
 
+import numpy as np
 import torch
 
 from .. import ops
 from ..cache.spec import StateSpec
 from ..ops.profile import section
-from .base import INIT_NORM_WEIGHT, LayerCache, ParamSpec, Part, StepContext, TensorSource
+from .base import INIT_NORM_WEIGHT, HostStep, LayerCache, ParamSpec, Part, StepContext, StepPlanner, TensorSource
+
+SEGMENT_FROM_TOKENS = 512     # a step whose longest entry has this many tokens gets the segments' work lists
+SEGMENT_UP_TO_BLOCKS = 2048   # ... and a layer walks in segments while whole entries would give fewer blocks than this
+
+
+class WalkSegments(StepPlanner):
+    """The work lists of the segmented walk, made once a step for all linear-attention layers: none
+    unless some entry is long (decode steps and short portions are walked whole)."""
+
+    key = "linear attention"
+
+    def plan(self, host: HostStep) -> Tuple[List[np.ndarray], dict]:
+        if not host.lens or max(host.lens) < SEGMENT_FROM_TOKENS:
+            empty = np.zeros(0, dtype=np.int32)
+            return [empty, empty], dict(n_segs=0)
+        segs, ents = ops.gla_segments(host.lens, host.cu_tokens)
+        return [segs.reshape(-1), ents.reshape(-1)], dict(n_segs=segs.shape[0])
+
+    def attach(self, ctx: StepContext, views: List[torch.Tensor], facts: dict) -> None:
+        ctx.extras[self.key] = (views[0], views[1]) if facts["n_segs"] else None
+
+
+_SEGMENTS = WalkSegments()
 
 
 class GatedLinearAttention(Part):
@@ -48,6 +72,9 @@ class GatedLinearAttention(Part):
         self.b_a2: Optional[torch.Tensor] = None      # float32 [heads * dk]
         self.w_norm: Optional[torch.Tensor] = None    # float32 [dv]
         self.w_o = None
+
+    def step_planners(self):
+        return (_SEGMENTS,)
 
     def cache_spec(self) -> StateSpec:
         return StateSpec(ops.gla_state_shape(self.nh, self.dk, self.dv), torch.float32)
@@ -102,7 +129,10 @@ class GatedLinearAttention(Part):
         state = cache.states[0] if cache.states else cache.state
         with section("recurrence", nbytes=lambda: 8 * ctx.n_entries * qk * self.dv + T * (width * (2 * qk + vv) + 4 * (qk + vv)),
                      flops=4.0 * T * qk * self.dv):
-            o = ops.gla_walk(proj, 0, qk, 2 * qk, alpha, self.dk ** -0.5, state, ctx, self.nh, self.dk, self.dv)
+            # a long entry alone in its step: walked in segments side by side (twice the sums on many times the blocks)
+            whole_blocks = ctx.n_entries * self.nh * ((self.dv + ops.GLA_STATE_COLS - 1) // ops.GLA_STATE_COLS)
+            segments = ctx.extras.get(_SEGMENTS.key) if whole_blocks < SEGMENT_UP_TO_BLOCKS else None
+            o = ops.gla_walk(proj, 0, qk, 2 * qk, alpha, self.dk ** -0.5, state, ctx, self.nh, self.dk, self.dv, segments=segments)
         with section("head norm + gate", nbytes=T * vv * (4 + 2 * width)):
             y = ops.head_norm_gate(o, self.w_norm, self.eps, self.nh, self.dv, ctx.act_dtype,
                                    proj if self.has_gate else None, 2 * qk + vv)

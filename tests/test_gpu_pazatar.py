@@ -202,6 +202,56 @@ def test_the_recurrence_walks_every_entry_from_its_slots_state(dtype, H, dk, dv,
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H, dk, dv, tau", [(2, 48, 64, 16.0), (1, 136, 20, 0.5), (3, 10, 24, 1.0)])
+def test_long_entries_walked_in_segments_side_by_side(dtype, H, dk, dv, tau):
+    """Two requests, each a long portion after a short one (so that the walk starts from a state that
+    is not zero): 700 and 129 tokens in one step, in segments of 128 (a last segment of 60 tokens, one of
+    a single token), against the plain recurrence; the states left in the slots against the whole walk's."""
+    from sharpinference_amd import ops
+
+    g = torch.Generator().manual_seed(dk * 7 + dv)
+    qk, vv, pad = H * dk, H * dv, 8
+    total = {"a": 705, "b": 132}
+    plan = [[("a", 5), ("b", 3)], [("b", 129), ("a", 700)]]
+    slot_of = {"a": 1, "b": 0}
+    proj = {r: torch.randn(n, pad + 2 * qk + vv, generator=g).to(DT[dtype]) for r, n in total.items()}
+    z = {r: torch.randn(n, qk, generator=g) * 2 + 2.0 for r, n in total.items()}
+    bias = torch.randn(qk, generator=g)
+    states = {}
+    outs = {}
+    for how in ("whole", "segments"):
+        state = torch.zeros(2, *ops.gla_state_shape(H, dk, dv), device=DEV)
+        got = {r: [] for r in total}
+        at = {r: 0 for r in total}
+        for step in plan:
+            lens = [n for _, n in step]
+            ctx = _Step(lens, [at[r] for r, _ in step], [slot_of[r] for r, _ in step])
+            rows = torch.cat([proj[r][at[r]:at[r] + n] for r, n in step]).to(DEV)
+            decays = ops.gla_decays(torch.cat([z[r][at[r]:at[r] + n] for r, n in step]).to(DEV), bias.to(DEV), tau)
+            segments = None
+            if how == "segments" and max(lens) > 128:
+                segs, ents = ops.gla_segments(lens, ctx.cu_tokens.cpu().numpy())
+                assert segs.shape == (8, 4) and ents.tolist() == [[0, 2], [2, 6]] and segs[1].tolist() == [0, 128, 1, 1]
+                segments = (torch.from_numpy(segs).to(DEV), torch.from_numpy(ents).to(DEV))
+            o = ops.gla_walk(rows, pad, pad + qk, pad + 2 * qk, decays, dk ** -0.5, state, ctx, H, dk, dv, segments=segments)
+            i = 0
+            for r, n in step:
+                got[r].append(o[i:i + n].cpu())
+                i += n
+                at[r] += n
+        outs[how] = {r: torch.cat(v) for r, v in got.items()}
+        states[how] = ops.gla_state_matrices(state, dk, dv).cpu()
+    for r, n in total.items():
+        p = proj[r].double()
+        alpha = torch.exp(torch.nn.functional.logsigmoid(z[r].double() + bias.double()) / tau).reshape(n, H, dk)
+        want = P.gated_recurrence(p[:, pad:pad + qk].reshape(n, H, dk) * dk ** -0.5, p[:, pad + qk:pad + 2 * qk].reshape(n, H, dk),
+                                  p[:, pad + 2 * qk:].reshape(n, H, dv), alpha)
+        assert _rel_rms(outs["segments"][r], want.reshape(n, -1)) < 3e-6, r
+        assert _rel_rms(outs["whole"][r], want.reshape(n, -1)) < 3e-6, r
+    assert _rel_rms(states["segments"].reshape(2, -1), states["whole"].reshape(2, -1)) < 3e-6
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("T, N, rank, tau", [(1, 20, 5, 3.0), (19, 288, 16, 16.0), (70, 520, 64, 0.5), (9, 40, 256, 1.0)])
 def test_decays_from_the_narrow_middle_of_their_projection(dtype, T, N, rank, tau):
     from sharpinference_amd import ops
@@ -511,6 +561,35 @@ def test_whole_prompts_portions_and_decoding_agree_with_the_plain_model(model_di
     assert eng.runner.graph_replays > 0                           # decode steps ran from graphs, states and all
     eng.cache.check_invariants()
     assert not eng.cache.requests
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["odd", "wide"])
+def test_a_long_prompt_is_walked_in_segments_and_agrees_with_its_portions(model_dirs, name, dtype, monkeypatch):
+    """700 tokens in one step: the linear-attention layers walk them in segments of 128 side by side;
+    the same tokens in portions of 100 are walked whole, portion by portion."""
+    from sharpinference_amd import ops
+
+    calls = {"segments": 0, "whole": 0}
+    walk = ops.gla_walk
+
+    def counted(*a, segments=None, **kw):
+        calls["segments" if segments is not None else "whole"] += 1
+        return walk(*a, segments=segments, **kw)
+
+    monkeypatch.setattr(ops, "gla_walk", counted)
+    d = model_dirs[name]
+    toks = _tokens(700, CONFIGS[name]["vocab"], 8)
+    eng = _engine(d, dtype, kv_tokens=2048)
+    whole = _run(eng, {"w": toks}, [[("w", 700)]])
+    assert calls["segments"] > 0 and calls["whole"] == 0
+    _check(d, dtype, {"w": toks}, whole, f"{name} {dtype} 700 tokens at once")
+    calls["segments"] = 0
+    parts = _run(eng, {"p": toks}, [[("p", 100)] for _ in range(7)])
+    assert calls["segments"] == 0 and calls["whole"] > 0
+    _check(d, dtype, {"p": toks}, parts, f"{name} {dtype} 700 tokens in portions")
+    if dtype == "float32":
+        assert _rel_rms(whole["w"], parts["p"]) < 1e-5
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
