@@ -244,7 +244,7 @@ __global__ __launch_bounds__(2 * kWave) void gla_walk_kernel(
       };
       if (nt == kStage) {
         // a full stage, unrolled: the LDS reads of the tokens ahead are requested while this one is summed
-#pragma unroll
+#pragma unroll 2
         for (int tt = 0; tt < kStage; ++tt) one_token(tt);
       } else {
         for (int tt = 0; tt < nt; ++tt) one_token(tt);
