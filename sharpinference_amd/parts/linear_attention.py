@@ -68,7 +68,7 @@ class GatedLinearAttention(Part):
         self.graph_safe = True         # entries and their state slots are read from the step's device arrays
         self.w_in = None               # [q | k | v | g] rows: one product of the input
         self.w_a1 = None               # (a product of its own: a few rows more spoil the large product's shape)
-        self.w_a2: Optional[torch.Tensor] = None      # [heads * dk, rank], row-major
+        self.w_a2: Optional[torch.Tensor] = None      # float32 [heads * dk, rank], row-major
         self.b_a2: Optional[torch.Tensor] = None      # float32 [heads * dk]
         self.w_norm: Optional[torch.Tensor] = None    # float32 [dv]
         self.w_o = None
@@ -106,7 +106,9 @@ class GatedLinearAttention(Part):
             o += p.shape[0]
         self.w_in = ops.pack_weight(fused)
         self.w_a1 = ops.pack_weight(source.get(prefix + n["a1"]))
-        self.w_a2 = source.get(prefix + n["a2"]).to(dt).contiguous()
+        # the second decay matrix in float whatever the activations are stored as: the decays' logits are then
+        # float sums over float values (a narrow middle rounded to bfloat16 would shift every decay of a token)
+        self.w_a2 = source.get(prefix + n["a2"]).float().contiguous()
         self.b_a2 = source.get(prefix + n["a2_bias"]).float().contiguous()
         self.w_norm = source.get(prefix + n["norm"]).float().contiguous()
         self.w_o = ops.pack_weight(source.get(prefix + n["o"]))
@@ -121,8 +123,8 @@ class GatedLinearAttention(Part):
         with section("q|k|v|g", nbytes=width * n_in * (self.hidden + T) + width * T * self.hidden, flops=2.0 * T * self.hidden * n_in):
             proj = ops.linear(x, self.w_in, ctx.act_dtype)
         with section("decays", nbytes=width * self.rank * (self.hidden + T + qk) + 4 * T * qk, flops=2.0 * T * self.rank * (self.hidden + qk)):
-            a1 = ops.linear(x, self.w_a1, ctx.act_dtype)
-            if T <= self.FUSED_DECAY_TOKENS and self.rank <= ops.GLA_FUSED_DECAY_MAX_RANK and a1.dtype == self.w_a2.dtype:
+            a1 = ops.linear(x, self.w_a1, torch.float32)
+            if T <= self.FUSED_DECAY_TOKENS and self.rank <= ops.GLA_FUSED_DECAY_MAX_RANK:
                 alpha = ops.gla_decays_from_middle(a1, 0, self.rank, self.w_a2, self.b_a2, self.tau)     # few tokens: one kernel
             else:
                 alpha = ops.gla_decays(ops.linear(a1, self.w_a2, torch.float32), self.b_a2, self.tau)
